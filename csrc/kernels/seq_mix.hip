@@ -1,0 +1,150 @@
+// Row kernels of the residual stream for models with per-sequence carried state and a depth-mixed stream:
+//
+//   embed_rows       x = table[token] (also the first entry of the layer history)
+//   token_shift      h = x + (x_prev - x) * mu: x_prev is the row above inside a step's run of tokens, the
+//                    sequence's carried row (state slot) at the start of a run, zeros at position 0
+//   add_layer_norm   x += layer_norm(delta) * w  (mean / variance / sum in fp32), optionally saving the rows that
+//                    become a sequence's carried state, appending the result to the layer history and replacing
+//                    x by the history's weighted sum, and writing the activation-dtype copy the next GEMM reads
+//   layer_norm       plain layer norm of gathered rows (the model's last norm)
+//
+// One 256-thread workgroup per row; columns strided over the threads (coalesced), any width.  The statistics
+// are two block reductions over the delta row (mean, then the squared deviations), so the variance is the
+// mean of squared deviations exactly as defined, not E[x^2] - E[x]^2.
+#include "common.h"
+#include "latent_launchers.h"
+
+namespace {
+
+constexpr int NT = 256;
+
+template <typename T>
+__global__ __launch_bounds__(NT) void embed_rows_kernel(const int* __restrict__ ids, const int* __restrict__ src,
+                                                        const int* __restrict__ prev, const T* __restrict__ table,
+                                                        float* __restrict__ x, float* __restrict__ hist0, int d) {
+  const int row = blockIdx.x;
+  const int sr = src ? src[row] : -1;
+  const long long tok = sr >= 0 ? prev[sr] : ids[row];
+  const T* t = table + tok * d;
+  for (int c = threadIdx.x; c < d; c += NT) {
+    const float v = (float)t[c];
+    x[(long long)row * d + c] = v;
+    hist0[(long long)row * d + c] = v;
+  }
+}
+
+template <typename T>
+__global__ __launch_bounds__(NT) void token_shift_kernel(const float* __restrict__ x, const T* __restrict__ mu,
+                                                         const int* __restrict__ prev_row,
+                                                         const float* __restrict__ state, long long state_stride,
+                                                         T* __restrict__ h, int d) {
+  const int row = blockIdx.x;
+  const int pr = prev_row[row];
+  const float* p = pr >= 0 ? x + (long long)pr * d : (pr == -1 ? nullptr : state + (long long)(-(pr + 2)) * state_stride);
+  for (int c = threadIdx.x; c < d; c += NT) {
+    const float xv = x[(long long)row * d + c];
+    const float pv = p ? p[c] : 0.f;
+    h[(long long)row * d + c] = (T)(xv + (pv - xv) * (float)mu[c]);
+  }
+}
+
+template <typename T, typename TD>
+__global__ __launch_bounds__(NT) void add_layer_norm_kernel(const TD* __restrict__ delta, const T* __restrict__ w,
+                                                            float eps, float* __restrict__ x,
+                                                            const int* __restrict__ save, float* __restrict__ state,
+                                                            long long state_stride, float* __restrict__ hist,
+                                                            long long hist_stride, const float* __restrict__ coef,
+                                                            int hist_idx, T* __restrict__ out_act, int d) {
+  __shared__ float scratch[NT / 64];
+  const int row = blockIdx.x;
+  const TD* dr = delta + (long long)row * d;
+  float sum = 0.f;
+  for (int c = threadIdx.x; c < d; c += NT) sum += (float)dr[c];
+  const float mean = block_sum<NT>(sum, scratch) / (float)d;
+  float sq = 0.f;
+  for (int c = threadIdx.x; c < d; c += NT) {
+    const float v = (float)dr[c] - mean;
+    sq += v * v;
+  }
+  const float rstd = 1.f / sqrtf(block_sum<NT>(sq, scratch) / (float)d + eps);
+  const int sv = save ? save[row] : -1;
+  for (int c = threadIdx.x; c < d; c += NT) {
+    const long long o = (long long)row * d + c;
+    const float xo = x[o];
+    if (sv >= 0) state[(long long)sv * state_stride + c] = xo;
+    float xn = xo + ((float)dr[c] - mean) * rstd * (float)w[c];
+    if (hist) {
+      hist[(long long)hist_idx * hist_stride + o] = xn;
+      float m = coef[hist_idx] * xn;
+      for (int j = 0; j < hist_idx; ++j) m += coef[j] * hist[(long long)j * hist_stride + o];
+      xn = m;
+    }
+    x[o] = xn;
+    if (out_act) out_act[o] = (T)xn;
+  }
+}
+
+template <typename T>
+__global__ __launch_bounds__(NT) void layer_norm_kernel(const float* __restrict__ x, const long long* __restrict__ rows,
+                                                        const T* __restrict__ w, float eps, T* __restrict__ out, int d) {
+  __shared__ float scratch[NT / 64];
+  const int i = blockIdx.x;
+  const float* xr = x + (rows ? rows[i] : (long long)i) * d;
+  float sum = 0.f;
+  for (int c = threadIdx.x; c < d; c += NT) sum += xr[c];
+  const float mean = block_sum<NT>(sum, scratch) / (float)d;
+  float sq = 0.f;
+  for (int c = threadIdx.x; c < d; c += NT) {
+    const float v = xr[c] - mean;
+    sq += v * v;
+  }
+  const float rstd = 1.f / sqrtf(block_sum<NT>(sq, scratch) / (float)d + eps);
+  for (int c = threadIdx.x; c < d; c += NT) out[(long long)i * d + c] = (T)((xr[c] - mean) * rstd * (float)w[c]);
+}
+
+}  // namespace
+
+void launch_embed_rows(const int* ids, const int* src, const int* prev, const void* table, float* x, float* hist0,
+                       int T, int d, int f32, hipStream_t s) {
+  if (T <= 0) return;
+  if (f32)
+    embed_rows_kernel<float><<<T, NT, 0, s>>>(ids, src, prev, (const float*)table, x, hist0, d);
+  else
+    embed_rows_kernel<bf16><<<T, NT, 0, s>>>(ids, src, prev, (const bf16*)table, x, hist0, d);
+}
+
+void launch_token_shift(const float* x, const void* mu, const int* prev_row, const float* state, long long state_stride,
+                        void* h, int T, int d, int f32, hipStream_t s) {
+  if (T <= 0) return;
+  if (f32)
+    token_shift_kernel<float><<<T, NT, 0, s>>>(x, (const float*)mu, prev_row, state, state_stride, (float*)h, d);
+  else
+    token_shift_kernel<bf16><<<T, NT, 0, s>>>(x, (const bf16*)mu, prev_row, state, state_stride, (bf16*)h, d);
+}
+
+void launch_add_layer_norm(const void* delta, int delta_f32, const void* w, float eps, float* x, const int* save,
+                           float* state, long long state_stride, float* hist, long long hist_stride, const float* coef,
+                           int hist_idx, void* out_act, int T, int d, int f32, hipStream_t s) {
+  if (T <= 0) return;
+  if (f32)
+    add_layer_norm_kernel<float, float><<<T, NT, 0, s>>>((const float*)delta, (const float*)w, eps, x, save, state,
+                                                        state_stride, hist, hist_stride, coef, hist_idx,
+                                                        (float*)out_act, d);
+  else if (delta_f32)
+    add_layer_norm_kernel<bf16, float><<<T, NT, 0, s>>>((const float*)delta, (const bf16*)w, eps, x, save, state,
+                                                       state_stride, hist, hist_stride, coef, hist_idx,
+                                                       (bf16*)out_act, d);
+  else
+    add_layer_norm_kernel<bf16, bf16><<<T, NT, 0, s>>>((const bf16*)delta, (const bf16*)w, eps, x, save, state,
+                                                      state_stride, hist, hist_stride, coef, hist_idx, (bf16*)out_act,
+                                                      d);
+}
+
+void launch_layer_norm(const float* x, const long long* rows, const void* w, float eps, void* out, int n, int d,
+                       int f32, hipStream_t s) {
+  if (n <= 0) return;
+  if (f32)
+    layer_norm_kernel<float><<<n, NT, 0, s>>>(x, rows, (const float*)w, eps, (float*)out, d);
+  else
+    layer_norm_kernel<bf16><<<n, NT, 0, s>>>(x, rows, (const bf16*)w, eps, (bf16*)out, d);
+}

@@ -41,6 +41,11 @@ ROCM = os.environ.get("ROCM_PATH", "/opt/rocm")
 HIPCC = os.path.join(ROCM, "bin", "hipcc")
 
 KERNEL_SO = os.path.join(PKG, "_C.so")
+LATENT_SO = os.path.join(PKG, "_C_latent.so")
+# the kernels of the latent-attention / carried-state / clamped-GLU model family and their op bindings: a library of
+# their own, so a process that serves only such a model builds (and loads) these three translation units
+LATENT_KERNELS = ("seq_mix.hip", "latent_attention.hip", "glu_moe.hip")
+LATENT_BINDINGS = ("latent_ops.cpp",)
 NET_SO = os.path.join(PKG, "net", "_native.so")
 RUNTIME_SO = os.path.join(PKG, "runtime", "_runtime.so")
 
@@ -90,6 +95,8 @@ HIP_FLAGS = [
     "-ffp-contract=fast",
     "-munsafe-fp-atomics",
     "-Wno-unused-result",
+    # no packed-fp32 instruction selection (v_pk_*_f32): scalar fp32 code only
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
 ]
 
 
@@ -97,7 +104,7 @@ def build_kernels(verbose: bool = False, force: bool = False) -> str:
     os.makedirs(OBJ, exist_ok=True)
     kdir = os.path.join(CSRC, "kernels")
     headers = glob.glob(os.path.join(kdir, "*.h")) + glob.glob(os.path.join(kdir, "*.cuh"))
-    sources = sorted(glob.glob(os.path.join(kdir, "*.hip")))
+    sources = sorted(s for s in glob.glob(os.path.join(kdir, "*.hip")) if os.path.basename(s) not in LATENT_KERNELS)
     tinc, tlib, abi = _torch_paths()
     jobs = []
     objs = []
@@ -107,7 +114,8 @@ def build_kernels(verbose: bool = False, force: bool = False) -> str:
         if force or _newer(obj, [src] + headers):
             cmd = [HIPCC, "-c", src, "-o", obj, "-I", kdir] + HIP_FLAGS
             jobs.append(cmd)
-    for bsrc in sorted(glob.glob(os.path.join(CSRC, "bindings", "*.cpp"))):
+    for bsrc in sorted(b for b in glob.glob(os.path.join(CSRC, "bindings", "*.cpp"))
+                       if os.path.basename(b) not in LATENT_BINDINGS):
         bobj = os.path.join(OBJ, "bind_" + os.path.basename(bsrc) + ".o")
         objs.append(bobj)
         if force or _newer(bobj, [bsrc] + headers):
@@ -128,6 +136,41 @@ def build_kernels(verbose: bool = False, force: bool = False) -> str:
         ]
         _run(cmd, verbose)
     return KERNEL_SO
+
+
+def build_latent(verbose: bool = False, force: bool = False) -> str:
+    """csrc/kernels/{seq_mix,latent_attention,glu_moe}.hip + csrc/bindings/latent_ops.cpp -> symmetry_amd/_C_latent.so
+    (``torch.ops.symmetry_amd_latent``)."""
+    os.makedirs(OBJ, exist_ok=True)
+    kdir = os.path.join(CSRC, "kernels")
+    headers = [os.path.join(kdir, "common.h"), os.path.join(kdir, "latent_launchers.h")]
+    tinc, tlib, abi = _torch_paths()
+    jobs, objs = [], []
+    for name in LATENT_KERNELS:
+        src, obj = os.path.join(kdir, name), os.path.join(OBJ, name + ".o")
+        objs.append(obj)
+        if force or _newer(obj, [src] + headers):
+            jobs.append([HIPCC, "-c", src, "-o", obj, "-I", kdir] + HIP_FLAGS)
+    for name in LATENT_BINDINGS:
+        src, obj = os.path.join(CSRC, "bindings", name), os.path.join(OBJ, "bind_" + name + ".o")
+        objs.append(obj)
+        if force or _newer(obj, [src] + headers):
+            cmd = [HIPCC, "-c", src, "-o", obj, "-I", kdir, "-O2", "-std=c++17", "-fPIC", f"--offload-arch={ARCH}",
+                   "-D__HIP_PLATFORM_AMD__=1", "-DUSE_ROCM=1", f"-D_GLIBCXX_USE_CXX11_ABI={abi}",
+                   "-DTORCH_EXTENSION_NAME=_C_latent", "-Wno-unused-result", "-Wno-deprecated-declarations"]
+            for i in tinc:
+                cmd += ["-isystem", i]
+            jobs.append(cmd)
+    if jobs:
+        with cf.ThreadPoolExecutor(_jobs()) as ex:
+            list(ex.map(lambda c: _run(c, verbose), jobs))
+    if force or jobs or _newer(LATENT_SO, objs):
+        tmp = LATENT_SO + f".{os.getpid()}.tmp"  # atomic: two first-use builds may race
+        _run([HIPCC, "-shared", "-o", tmp] + objs + [f"--offload-arch={ARCH}", "-L", tlib, "-lc10", "-lc10_hip",
+                                                      "-ltorch_cpu", "-ltorch_hip", "-ltorch", f"-Wl,-rpath,{tlib}"],
+             verbose)
+        os.replace(tmp, LATENT_SO)
+    return LATENT_SO
 
 
 # --------------------------------------------------------------------------------------
@@ -207,6 +250,7 @@ def build_all(verbose: bool = False, force: bool = False):
     net = build_net(verbose, force)
     build_runtime(verbose, force)
     ker = build_kernels(verbose, force)
+    build_latent(verbose, force)
     return ker, net
 
 
@@ -218,6 +262,8 @@ if __name__ == "__main__":
         print(build_net(verbose, force))
     if not what or "kernels" in what:
         print(build_kernels(verbose, force))
+    if not what or "latent" in what:
+        print(build_latent(verbose, force))
     if not what or "runtime" in what:
         print(build_runtime(verbose, force))
     if "selftest" in what:

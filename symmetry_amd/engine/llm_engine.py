@@ -24,12 +24,12 @@ from dataclasses import dataclass, field
 
 import torch
 
+from ..models import model_class
 from ..models.config import ModelConfig, resolve
-from ..models.transformer import KVCache, TransformerLM
 from ..models.weights import ModelWeights, ShardSpec, load_hf_weights, random_weights
 from ..utils.metrics import EngineMetrics
 from .model_runner import MAX_DECODE_ROWS, ModelRunner
-from .scheduler import BlockManager, Scheduler, SchedulerConfig
+from .scheduler import BlockManager, Scheduler, SchedulerConfig, StateSlotManager
 from .sequence import SamplingParams, Sequence, SeqStatus
 from .tokenizer import IncrementalDetokenizer, load_tokenizer
 
@@ -68,6 +68,8 @@ class EngineConfig:
     arrival_quiet_us: int = int(os.environ.get("SYMMETRY_ARRIVAL_QUIET_US", "300"))
     arrival_window_us: int = int(os.environ.get("SYMMETRY_ARRIVAL_WINDOW_US", "2000"))
     model_config: ModelConfig | None = None
+    # activation / weight dtype: "bfloat16" (serving) or "float32" (true 32-bit everywhere; models that support it)
+    dtype: str = "bfloat16"
 
     @classmethod
     def from_provider(cls, cfg: dict, **overrides) -> "EngineConfig":
@@ -83,7 +85,7 @@ class EngineConfig:
              "useGraphs": "use_graphs", "numKvBlocks": "num_kv_blocks", "decodeWeights": "decode_weights",
              "prefillChunk": "mixed_prefill_tokens",
              "enablePrefixCaching": "enable_prefix_caching", "burstSplitTokens": "burst_split_tokens",
-             "arrivalQuietUs": "arrival_quiet_us", "arrivalWindowUs": "arrival_window_us"}
+             "arrivalQuietUs": "arrival_quiet_us", "arrivalWindowUs": "arrival_window_us", "dtype": "dtype"}
         for k, attr in m.items():
             if cfg.get(k) is not None:
                 cur, val = getattr(ec, attr), cfg[k]
@@ -128,6 +130,12 @@ class LLMEngine:
         self.metrics = EngineMetrics()
         shard = ShardSpec(cfg.tp_rank, cfg.tp_size, cfg.ep_rank, cfg.ep_size)
         t0 = time.perf_counter()
+        cls = model_class(mcfg)
+        if cfg.dtype not in ("bfloat16", "float32"):
+            raise ValueError(f"dtype {cfg.dtype!r}: bfloat16 or float32")
+        dtype = torch.float32 if cfg.dtype == "float32" else torch.bfloat16
+        if dtype == torch.float32 and not getattr(cls, "has_seq_state", False):
+            raise ValueError(f"{mcfg.name}: this model family is served in bfloat16 only")
         if cfg.weights == "random":
             mode = cfg.weight_init
             if mode == "auto":
@@ -139,16 +147,21 @@ class LLMEngine:
         self.load_time = time.perf_counter() - t0
         # what the KV cache needs for the admission limit at full context: the optional weight copies (preshuffled decode
         # / expert streams) are sized from the HBM left after it, never from the KV cache's share
-        per_block = mcfg.kv_bytes_per_token() // cfg.tp_size * cfg.block_size
+        self._kv_elem = 4 if dtype == torch.float32 else 2
+        per_block = mcfg.kv_bytes_per_token(self._kv_elem) // cfg.tp_size * cfg.block_size
         kv_need = (cfg.num_kv_blocks or -(-cfg.max_num_seqs * max_model_len // cfg.block_size)) * per_block
-        self.model = TransformerLM(weights, self.device, tp_comm=tp_comm, ep_comm=ep_comm,
-                                   max_decode_ctx=max_model_len, decode_weights=cfg.decode_weights,
-                                   kv_reserve_bytes=kv_need)
+        extra = {"dtype": dtype} if getattr(cls, "has_seq_state", False) else {}
+        self.model = cls(weights, self.device, tp_comm=tp_comm, ep_comm=ep_comm, max_decode_ctx=max_model_len,
+                         decode_weights=cfg.decode_weights, kv_reserve_bytes=kv_need, **extra)
         self.tokenizer = load_tokenizer(mcfg, cfg.tokenizer or (cfg.weights if cfg.weights != "random" else None))
         nb = cfg.num_kv_blocks or self._auto_blocks(max_model_len)
-        self.kv = KVCache(mcfg.num_layers, nb, mcfg.num_kv_heads // cfg.tp_size, mcfg.head_dim, cfg.block_size,
-                          self.device)
-        self.blocks = BlockManager(nb, cfg.block_size, prefix_caching=cfg.enable_prefix_caching)
+        num_seqs = min(cfg.max_num_seqs, self._max_decode_rows(mcfg))
+        # the model builds its own cache: paged K/V (Llama / Mixtral), or paged latents + one state slot per live
+        # sequence (models with carried state; their cached blocks alone do not restore a prefix, so no prefix caching)
+        self.kv = self.model.make_cache(nb, cfg.block_size, num_seqs)
+        self.slots = StateSlotManager(num_seqs) if self.model.has_seq_state else None
+        self.blocks = BlockManager(nb, cfg.block_size,
+                                   prefix_caching=cfg.enable_prefix_caching and not self.model.has_seq_state)
         if self.device.type != "cpu":
             extra = self.model.extra_weight_bytes()
             print(f"symmetry: {mcfg.name} weights {weights.nbytes() / 1e9:.1f} GB + layout copies {extra / 1e9:.1f} GB; "
@@ -159,7 +172,7 @@ class LLMEngine:
                             max_num_batched_tokens=cfg.max_num_batched_tokens, max_model_len=max_model_len,
                             mixed_prefill_tokens=cfg.mixed_prefill_tokens,
                             burst_split_tokens=cfg.burst_split_tokens),
-            self.blocks)
+            self.blocks, self.slots)
         self.runner = ModelRunner(self.model, self.kv, self.scheduler.cfg.max_num_seqs, max_model_len,
                                   use_graphs=cfg.use_graphs and self._graph_safe(tp_comm, ep_comm),
                                   tp_rank=cfg.tp_rank, tp_size=cfg.tp_size, cpu_group=cpu_group,
@@ -194,10 +207,10 @@ class LLMEngine:
             if os.path.exists(path):
                 import json
 
-                from ..models.config import from_hf_config
+                from ..models.config import from_config_json
 
                 with open(path) as f:
-                    return from_hf_config(json.load(f), name=cfg.model)
+                    return from_config_json(json.load(f), name=cfg.model)
         return resolve(cfg.model)
 
     def _max_decode_rows(self, mcfg: ModelConfig) -> int:
@@ -221,7 +234,7 @@ class LLMEngine:
         return True
 
     def _auto_blocks(self, max_model_len: int) -> int:
-        per_block = self.model_cfg.kv_bytes_per_token() // self.cfg.tp_size * self.cfg.block_size
+        per_block = self.model_cfg.kv_bytes_per_token(self._kv_elem) // self.cfg.tp_size * self.cfg.block_size
         if self.device.type == "cpu":
             want = (self.cfg.max_num_seqs * max_model_len) // self.cfg.block_size + 8
             return max(16, min(want, (1 << 30) // per_block))
@@ -307,6 +320,42 @@ class LLMEngine:
             self.metrics.on_abort()
         if seq is not None and entry is not None:
             self._emit(entry[2], RequestOutput(request_id, [], "", True, "abort", seq=seq))
+
+    # ---- replayed steps (trace runner) -----------------------------------------------------------
+    def replay_step(self, entries: list, end: list = ()) -> torch.Tensor | None:
+        """Run one step whose content the caller dictates and return the wanted logits.
+
+        ``entries``: [(request id, next token ids, offsets among them whose logits are wanted)]; a request is admitted
+        at its first entry and may skip steps; ``end``: requests finished after this step (their cache blocks and
+        state slot go back to the pools).  The step takes the engine's ordinary route -- Scheduler (block growth,
+        state slots) -> ModelRunner.launch (packed metadata, decode hipGraphs) -> model.forward -- with sampling off.
+        Returns fp32 logits [wanted, vocab] on the host in entry order, or None if nothing is wanted."""
+        if self._inflight is not None:
+            raise RuntimeError("replay_step while a pipelined decode step is in flight")
+        given = []
+        with self.lock:
+            for rid, tokens, want in entries:
+                ent = self.requests.get(rid)
+                if ent is None:
+                    seq = Sequence(rid, [], SamplingParams(max_tokens=1), eos_ids=())
+                    self.requests[rid] = ent = (seq, None, None)
+                seq = ent[0]
+                seq.prompt_ids.extend(int(t) for t in tokens)
+                given.append((seq, len(tokens), want))
+            batch = self.scheduler.schedule_given(given) if given else None
+        logits = None
+        if batch is not None:
+            fl = self._launch(batch, None)
+            if "failed" in fl:
+                raise RuntimeError(f"replayed step failed: {fl['failed'][0].error}")
+            self.runner.wait(fl["handle"])
+            logits = fl["handle"].get("logits_host")
+        with self.lock:
+            for rid in end:
+                ent = self.requests.pop(rid, None)
+                if ent is not None:
+                    self.scheduler.finish(ent[0], SeqStatus.FINISHED_STOPPED)
+        return logits
 
     def has_unfinished(self) -> bool:
         fl = self._inflight

@@ -69,7 +69,8 @@ def _seq_seed(seed: int, n_out: int) -> int:
 class _Layout:
     """Offsets of the packed int32 metadata buffer."""
 
-    def __init__(self, T: int, nseq: int, max_blocks: int, prefill: bool, ntiles: int = 0):
+    def __init__(self, T: int, nseq: int, max_blocks: int, prefill: bool, ntiles: int = 0, state: bool = False,
+                 nlog: int = 0):
         off = 0
 
         def take(n):
@@ -99,6 +100,17 @@ class _Layout:
             if off % 2:
                 take(1)
             self.last = take(2 * nseq)
+        # models with per-sequence state: previous row / state slot of every token row, the slot a sequence's last
+        # row is saved to, and the batch index of every row
+        self.state, self.nlog = state, nlog
+        if state:
+            self.prev = take(T)
+            self.save = take(T)
+            self.rowseq = take(T)
+        if nlog:  # token rows whose logits the caller wants (int64)
+            if off % 2:
+                take(1)
+            self.logrows = take(2 * nlog)
         self.size = off + (off % 2)
 
     def views(self, buf: torch.Tensor) -> dict:
@@ -119,6 +131,12 @@ class _Layout:
             v["cu_q"] = buf[self.cu:self.cu + self.nseq + 1]
             v["tiles"] = buf[self.tiles:self.tiles + 2 * self.ntiles].view(self.ntiles, 2)
             v["last_idx"] = buf[self.last:self.last + 2 * self.nseq].view(torch.int64)
+        if self.state:
+            v["prev_row"] = buf[self.prev:self.prev + self.T]
+            v["save_slot"] = buf[self.save:self.save + self.T]
+            v["row_seq"] = buf[self.rowseq:self.rowseq + self.T]
+        if self.nlog:
+            v["logit_rows"] = buf[self.logrows:self.logrows + 2 * self.nlog].view(torch.int64)
         return v
 
 
@@ -139,6 +157,7 @@ class ModelRunner:
         self.ctx_blocks = [b for b in self.ctx_blocks if b <= self.max_blocks]
         self.is_gpu = self.device.type != "cpu"
         self.use_graphs = use_graphs and self.is_gpu
+        self.seq_state = bool(getattr(model, "has_seq_state", False))
         # pad short prefills to the graph buckets (without use_graphs -- CPU tests -- they then run eagerly)
         self.prefill_graphs = self.use_graphs
         self.prefill_graph_replays = 0
@@ -225,6 +244,13 @@ class ModelRunner:
             x = seed * np.uint64(0x100000001B3) + nout * np.uint64(_SEED_MIX)
         x ^= x >> np.uint64(29)
         host[lay.seeds:lay.seeds + 2 * n] = x.view(np.int32)
+        if lay.state:  # one row per sequence: the previous token's row is the sequence's carried state
+            slot = np.fromiter((s.state_slot for s in seqs), np.int64, n)
+            host[lay.prev:lay.prev + T] = -1
+            host[lay.prev:lay.prev + n] = np.where(pos > 0, -(slot + 2), -1)
+            host[lay.save:lay.save + T] = -1
+            host[lay.save:lay.save + n] = slot
+            host[lay.rowseq:lay.rowseq + n] = np.arange(n)
 
     def _fill(self, lay: _Layout, host: np.ndarray, seqs, counts, prev_rows: dict | None = None) -> None:
         """Pack one step's metadata.  A decode row whose input token is still in flight (sampled by the
@@ -295,11 +321,22 @@ class ModelRunner:
             if lay.ntiles > len(tiles):  # padding tiles (graph buckets): row past every qlen -> workgroup exits
                 host[lay.tiles + 2 * len(tiles) + 1:lay.tiles + 2 * lay.ntiles:2] = _PAD_TILE_ROW
             host[lay.last:lay.last + 2 * lay.nseq] = np.maximum(cu[1:] - 1, 0).astype(np.int64).view(np.int32)
+        if lay.state:
+            host[lay.prev:lay.prev + T] = -1
+            host[lay.save:lay.save + T] = -1
+            r0 = 0
+            for i, (seq, n) in enumerate(zip(seqs, counts)):
+                # a run of n rows: the first reads the carried state (nothing at position 0), the others the row above
+                host[lay.prev + r0:lay.prev + r0 + n] = np.arange(r0 - 1, r0 + n - 1)
+                host[lay.prev + r0] = -1 if seq.num_computed == 0 else -(seq.state_slot + 2)
+                host[lay.save + r0 + n - 1] = seq.state_slot
+                host[lay.rowseq + r0:lay.rowseq + r0 + n] = i
+                r0 += n
 
     def _forward_batch(self, kind: str, lay: _Layout, dev: torch.Tensor, nseq: int, need_logits=False,
-                       filtered=False):
+                       filtered=False, sample=True):
         v = lay.views(dev)
-        return ForwardBatch(kind=kind, num_seqs=nseq, need_logits=need_logits, filtered=filtered, **v)
+        return ForwardBatch(kind=kind, num_seqs=nseq, need_logits=need_logits, filtered=filtered, sample=sample, **v)
 
     @staticmethod
     def _filtered(seqs) -> bool:
@@ -319,25 +356,39 @@ class ModelRunner:
         t0 = time.perf_counter()
         filt = int(self._filtered(seqs))
         nseq = len(seqs)
+        # logits the caller wants back (replayed steps): token rows of a prefill-kind step; a decode step returns
+        # every row's (the sampler's own logits) and the wanted sequences are picked on the host
+        want = batch.logit_offsets
+        log_rows, r0 = [], 0
+        if want is not None:
+            for n, offs in zip(counts, want):
+                log_rows.extend(r0 + o for o in offs)
+                r0 += n
+        need_logits = bool(log_rows) and batch.kind == "decode"
+        sample = any(batch.sample) if batch.sample else True
+        st = self.seq_state
         if batch.kind == "decode":
             bucket = self._bucket(nseq)
             need = max(len(s.block_table) for s in seqs)
-            lay = _Layout(bucket, bucket, self._ctx_bucket(need), prefill=False)
+            lay = _Layout(bucket, bucket, self._ctx_bucket(need), prefill=False, state=st)
             kind = KIND_DECODE
         else:
             T = sum(counts)
             max_blocks = max(len(s.block_table) for s in seqs)
-            shape = self._prefill_graph_shape(T, nseq, max_blocks, filt)
+            shape = self._prefill_graph_shape(T, nseq, max_blocks, filt) if not log_rows else None
             if shape is not None:
-                lay, kind = _Layout(*shape, prefill=True, ntiles=self._pad_tiles(shape[0], shape[1])), \
+                lay, kind = _Layout(*shape, prefill=True, ntiles=self._pad_tiles(shape[0], shape[1]), state=st), \
                     KIND_PREFILL_GRAPH
             else:
                 ntiles = sum((n + 63) // 64 for n in counts)
-                lay, kind = _Layout(T, nseq, max_blocks, prefill=True, ntiles=ntiles), KIND_PREFILL
+                lay, kind = _Layout(T, nseq, max_blocks, prefill=True, ntiles=ntiles, state=st,
+                                    nlog=len(log_rows)), KIND_PREFILL
         self._parity ^= 1
         host_t = self._host(lay.size, f"{batch.kind}{self._parity}")  # double-buffered: the previous
         host = host_t.numpy()                                          # step's H2D may still be queued
         self._fill(lay, host, seqs, counts, prev_rows)
+        if lay.nlog:
+            host[lay.logrows:lay.logrows + 2 * lay.nlog] = np.asarray(log_rows, dtype=np.int64).view(np.int32)
         if _DEBUG_PREFILL and batch.kind != "decode":  # the shape a prefill step's kernels see (bench diagnosis)
             bts = [b for s in seqs for b in s.block_table]
             print(f"symmetry: prefill step T={sum(counts)} seqs={nseq} new={list(counts)} "
@@ -348,9 +399,13 @@ class ModelRunner:
         if self.meta is not None:
             self._broadcast(header, host_t)
         t2 = time.perf_counter()
-        ids = self._run(header, host_t)
+        ids = self._run(header, host_t, nlog=lay.nlog, need_logits=need_logits, sample=sample)
         t3 = time.perf_counter()
         handle = {"nseq": nseq, "t0": t0}
+        if log_rows:
+            # (device tensor in the model's workspace: read it before the next launch overwrites it)
+            handle["logits"] = self.model.last_logits
+            handle["logit_pick"] = log_rows if need_logits else None
         if self.is_gpu:
             pin = self._host(max(ids.numel(), 1), f"ids_out{self._parity}")[:ids.numel()]
             if _native.available() and ids.is_contiguous():
@@ -383,6 +438,11 @@ class ModelRunner:
         else:
             ids = handle["ids"]
         self.timing["forward"] += time.perf_counter() - handle["t0"]
+        if "logits" in handle:
+            lg = handle.pop("logits")
+            pick = handle.pop("logit_pick")
+            lg = lg if pick is None else lg[torch.as_tensor(pick, device=lg.device)]
+            handle["logits_host"] = lg.float().cpu()
         return ids[:handle["nseq"]]
 
     @staticmethod
@@ -406,7 +466,9 @@ class ModelRunner:
         return Tb, nb, mb
 
     def _prefill_graphs_on(self) -> bool:
-        return self.prefill_graphs and PREFILL_GRAPH_TOKENS > 0 and self.tp_size == 1 and not self.model.cfg.is_moe
+        # (models with carried state keep prefill eager: their padded rows would need state-free metadata)
+        return (self.prefill_graphs and PREFILL_GRAPH_TOKENS > 0 and self.tp_size == 1 and not self.model.cfg.is_moe
+                and not self.seq_state)
 
     def _bucket(self, n: int) -> int:
         for b in self.buckets:
@@ -420,13 +482,14 @@ class ModelRunner:
                 return b
         raise ValueError(f"sequence needs {nblocks} blocks > max {self.max_blocks}")
 
-    def _run(self, header: np.ndarray, host_t: torch.Tensor) -> torch.Tensor:
+    def _run(self, header: np.ndarray, host_t: torch.Tensor, nlog: int = 0, need_logits: bool = False,
+             sample: bool = True) -> torch.Tensor:
         kind = "decode" if header[0] == KIND_DECODE else "prefill"
         T, nseq_l, max_blocks, ntiles, nseq, filt = (int(x) for x in header[1:HEADER_LEN])
-        lay = _Layout(T, nseq_l, max_blocks, prefill=kind == "prefill", ntiles=ntiles)
+        lay = _Layout(T, nseq_l, max_blocks, prefill=kind == "prefill", ntiles=ntiles, state=self.seq_state, nlog=nlog)
         if self.use_graphs and (kind == "decode" or header[0] == KIND_PREFILL_GRAPH):
             if kind == "decode":
-                key = (T, max_blocks, bool(filt))
+                key = (T, max_blocks, bool(filt)) + ((need_logits, sample) if need_logits or not sample else ())
                 self.graph_replays += 1
             else:
                 key = ("prefill", T, nseq_l, max_blocks, ntiles, bool(filt))
@@ -434,11 +497,13 @@ class ModelRunner:
             g = self.graphs.get(key)
             if g is None:
                 if kind == "decode":
-                    self._capture(T, max_blocks, bool(filt))
+                    self._capture(T, max_blocks, bool(filt), need_logits=need_logits, sample=sample)
                 else:
                     self._capture(T, max_blocks, bool(filt), prefill=lay)
                 g = self.graphs[key]
-            graph, dev, out, exec_ = g
+            graph, dev, out, exec_ = g[:4]
+            if need_logits:
+                self.model.last_logits = g[4]
             if exec_:
                 # H2D + hipGraphLaunch with the GIL held (torch's copy_ / replay() release it and the engine
                 # thread then waits for the event-loop thread: csrc/bindings/torch_ops.cpp, graph_launch)
@@ -454,24 +519,25 @@ class ModelRunner:
         else:
             dev = self.model.ws.get("meta." + kind, (lay.size,), torch.int32, self.device)
             dev.copy_(host_t[:lay.size], non_blocking=True)
-            fb = self._forward_batch(kind, lay, dev, nseq_l, filtered=bool(filt))
+            fb = self._forward_batch(kind, lay, dev, nseq_l, filtered=bool(filt), need_logits=need_logits, sample=sample)
             ids = self.model.forward(fb, self.kv)
         return ids
 
     # ------------------------------------------------------------------------------------------
-    def _capture(self, bucket: int, max_blocks: int, filtered: bool = False, prefill: _Layout | None = None) -> None:
+    def _capture(self, bucket: int, max_blocks: int, filtered: bool = False, prefill: _Layout | None = None,
+                 need_logits: bool = False, sample: bool = True) -> None:
         """Capture the decode forward for `bucket` rows and a `max_blocks`-wide block table, with or
         without the top-k / top-p resampler (largest first avoids workspace growth).  ``prefill``: capture
         that padded prefill layout instead (the warmup and capture run on all-padding metadata: no cache
         slot is written, every attention tile exits)."""
-        lay = prefill if prefill is not None else _Layout(bucket, bucket, max_blocks, prefill=False)
+        lay = prefill if prefill is not None else _Layout(bucket, bucket, max_blocks, prefill=False, state=self.seq_state)
         kind = "prefill" if prefill is not None else "decode"
         dev = torch.zeros(lay.size, dtype=torch.int32, device=self.device)
         host = self._host(lay.size, "capture")
         hn = host.numpy()
         self._fill(lay, hn, [], [])
         dev.copy_(host[:lay.size])
-        fb = self._forward_batch(kind, lay, dev, lay.nseq, filtered=filtered)
+        fb = self._forward_batch(kind, lay, dev, lay.nseq, filtered=filtered, need_logits=need_logits, sample=sample)
         # eager warmup: allocates workspace and loads kernels outside the capture
         s = torch.cuda.Stream()
         s.wait_stream(torch.cuda.current_stream())
@@ -492,9 +558,9 @@ class ModelRunner:
                 exec_ = int(g.raw_cuda_graph_exec())
             except Exception:  # noqa: BLE001 -- older torch: replay() it is
                 exec_ = 0
-        key = (bucket, max_blocks, filtered) if prefill is None else \
-            ("prefill", lay.T, lay.nseq, lay.max_blocks, lay.ntiles, filtered)
-        self.graphs[key] = (g, dev, out, exec_)
+        key = (bucket, max_blocks, filtered) + ((need_logits, sample) if need_logits or not sample else ()) \
+            if prefill is None else ("prefill", lay.T, lay.nseq, lay.max_blocks, lay.ntiles, filtered)
+        self.graphs[key] = (g, dev, out, exec_, getattr(self.model, "last_logits", None) if need_logits else None)
 
     def capture_all(self) -> float:
         """Rank 0: capture every (batch, context) decode graph; under TP each capture is mirrored by the

@@ -165,6 +165,33 @@ class BlockManager:
         seq.block_table = []
 
 
+class StateSlotManager:
+    """Slots of per-sequence model state (models that carry state from token to token besides the paged cache:
+    ``model.has_seq_state``).  A sequence holds one slot from admission until it finishes or is preempted; a
+    released slot is handed out again (its old content is never read: a sequence's first token reads no state)."""
+
+    def __init__(self, num_slots: int):
+        self.num_slots = num_slots
+        self.free = collections.deque(range(num_slots))
+
+    @property
+    def num_free(self) -> int:
+        return len(self.free)
+
+    def alloc(self, seq: Sequence) -> bool:
+        if seq.state_slot >= 0:
+            return True
+        if not self.free:
+            return False
+        seq.state_slot = self.free.popleft()
+        return True
+
+    def release(self, seq: Sequence) -> None:
+        if seq.state_slot >= 0:
+            self.free.append(seq.state_slot)
+            seq.state_slot = -1
+
+
 @dataclass
 class SchedulerConfig:
     max_num_seqs: int = 64
@@ -185,6 +212,8 @@ class ScheduledBatch:
     num_new_tokens: list            # tokens computed this step per sequence
     sample: list = field(default_factory=list)  # whether this step's sample is kept per sequence
     preempted: list = field(default_factory=list)
+    # per sequence, offsets among this step's tokens whose logits the caller wants back (replayed steps), or None
+    logit_offsets: list | None = None
 
     @property
     def num_tokens(self) -> int:
@@ -192,9 +221,10 @@ class ScheduledBatch:
 
 
 class Scheduler:
-    def __init__(self, cfg: SchedulerConfig, blocks: BlockManager):
+    def __init__(self, cfg: SchedulerConfig, blocks: BlockManager, slots: StateSlotManager | None = None):
         self.cfg = cfg
         self.blocks = blocks
+        self.slots = slots  # state slots of models with per-sequence state (None: the paged cache is all there is)
         self.waiting: collections.deque[Sequence] = collections.deque()
         self.running: list[Sequence] = []
         self._burst_rest = 0  # prompt tokens of a split burst left for the next step
@@ -211,6 +241,8 @@ class Scheduler:
     def finish(self, seq: Sequence, status: SeqStatus) -> None:
         seq.status = status
         self.blocks.release(seq)
+        if self.slots is not None:
+            self.slots.release(seq)
         if seq in self.running:
             self.running.remove(seq)
         else:
@@ -315,8 +347,12 @@ class Scheduler:
         # 2) admit waiting sequences
         while self.waiting and budget > 0 and len(self.running) < self.cfg.max_num_seqs:
             seq = self.waiting[0]
+            if self.slots is not None and seq.state_slot < 0 and not self.slots.num_free:
+                break
             if not take(seq):
                 break
+            if self.slots is not None:
+                self.slots.alloc(seq)
             self.waiting.popleft()
             seq.status = SeqStatus.RUNNING
             self.running.append(seq)
@@ -360,8 +396,35 @@ class Scheduler:
         b = self._schedule_decode()
         return b if b is not None and b.seqs else None
 
+    def schedule_given(self, entries: list) -> ScheduledBatch:
+        """A step whose content the caller dictates (trace replay): ``entries`` = [(sequence, tokens this step,
+        offsets of wanted logits)].  New sequences are admitted (state slot, running list); cache blocks grow
+        exactly as for a scheduled step.  A step of single tokens that all continue their sequences is a decode
+        step; anything else is the mixed / prefill kind, as ``schedule`` would form it."""
+        seqs, counts, want = [], [], []
+        for seq, n, offs in entries:
+            if n <= 0 or seq.num_computed + n > seq.num_tokens:
+                raise ValueError(f"{seq.request_id}: {n} tokens past its {seq.num_tokens - seq.num_computed} known ones")
+            if seq not in self.running:
+                if len(self.running) >= self.cfg.max_num_seqs or (self.slots is not None and not self.slots.alloc(seq)):
+                    raise MemoryError(f"{seq.request_id}: no free sequence slot ({self.cfg.max_num_seqs} live)")
+                try:
+                    self.waiting.remove(seq)
+                except ValueError:
+                    pass
+                seq.status = SeqStatus.RUNNING
+                self.running.append(seq)
+            self.blocks.grow(seq, seq.num_computed + n)
+            seqs.append(seq)
+            counts.append(n)
+            want.append(list(offs))
+        decode = all(n == 1 and s.num_computed > 0 for s, n in zip(seqs, counts))
+        return ScheduledBatch("decode" if decode else "prefill", seqs, counts, [False] * len(seqs), [], want)
+
     def _preempt(self, seq: Sequence) -> None:
         self.blocks.release(seq)
+        if self.slots is not None:
+            self.slots.release(seq)
         seq.num_computed = 0
         seq.prefix_checked = False
         seq.num_preemptions += 1

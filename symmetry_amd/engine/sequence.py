@@ -85,6 +85,7 @@ class Sequence:
     cache_scope: bytes = b""       # prefix-cache namespace (client identity)
     prefix_checked: bool = False   # the prefix cache was consulted for the current (fresh) KV state
     prefix_epoch: int = -1         # the prefix cache's size at that look (a grown cache is re-queried)
+    state_slot: int = -1           # slot of the model's per-sequence state (models with carried state), -1: none
 
     @property
     def token_ids(self) -> list:

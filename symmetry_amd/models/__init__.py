@@ -1,0 +1,14 @@
+"""Model families.  ``model_class(cfg)`` maps a configuration to the class that runs it."""
+
+
+def model_class(cfg):
+    family = getattr(cfg, "family", "llama")
+    if family == "bozevik":
+        from .bozevik import BozevikLM
+
+        return BozevikLM
+    if family == "llama":
+        from .transformer import TransformerLM
+
+        return TransformerLM
+    raise KeyError(f"no model class for family {family!r}")

@@ -13,6 +13,7 @@ from dataclasses import dataclass, field
 
 @dataclass(frozen=True)
 class ModelConfig:
+    family = "llama"  # which model class runs it (models.model_class); not a field
     name: str
     vocab_size: int
     hidden_size: int
@@ -61,6 +62,198 @@ class ModelConfig:
         return dataclasses.replace(self, **kw)
 
 
+# --------------------------------------------------------------------------------------------------
+# Bozevik: per-layer specs (every layer names its mixer and feed-forward), latent attention, clamped GLU / MoE
+# --------------------------------------------------------------------------------------------------
+@dataclass(frozen=True)
+class LatentMixerSpec:
+    """Attention through low-rank latents: queries via q_rank, keys / values via a cached kv_rank latent plus one
+    rotated key part of rot_dim shared by all heads.  ``kv_from``: the layer whose cache this layer attends
+    (it then has no down-projection of its own)."""
+    heads: int
+    dim: int            # unrotated query / key dims per head
+    rot_dim: int        # rotated dims per head (and of the shared key part)
+    vdim: int
+    kv_rank: int
+    q_rank: int
+    rot_base: float
+    rot_dims: int       # leading dims of the rotated part that turn (pairs 2i, 2i + 1)
+    scale: float
+    kv_from: int | None = None
+
+
+@dataclass(frozen=True)
+class GluSpec:
+    ff: int
+    limit: float
+
+
+@dataclass(frozen=True)
+class MoeSpec:
+    experts: int
+    top: int
+    expert: GluSpec
+    shared: GluSpec | None = None
+
+
+@dataclass(frozen=True)
+class LayerSpec:
+    type: str                       # mixer kind: "latent_attention"
+    mixer: LatentMixerSpec
+    mlp: GluSpec | MoeSpec | None = None
+
+
+@dataclass(frozen=True)
+class BozevikConfig:
+    family = "bozevik"
+    name: str
+    vocab_size: int
+    hidden_size: int
+    layers: tuple
+    norm_eps: float = 1e-6
+    logit_scale: float = 1.0
+    max_position: int = 131072
+    bos_token_id: int = 1
+    eos_token_ids: tuple = (2,)
+    chat_format: str = "llama3"
+    tie_embeddings = True
+    rope_scaling = None
+
+    @property
+    def num_layers(self) -> int:
+        return len(self.layers)
+
+    @property
+    def is_moe(self) -> bool:
+        return any(isinstance(layer.mlp, MoeSpec) for layer in self.layers)
+
+    def cache_layers(self) -> list:
+        """Layers that own a cache plane (a down-projection of their own), in order."""
+        return [i for i, layer in enumerate(self.layers) if layer.mixer.kv_from is None]
+
+    def num_params(self) -> int:
+        d, n = self.hidden_size, self.vocab_size * self.hidden_size + self.hidden_size
+        for i, layer in enumerate(self.layers):
+            m = layer.mixer
+            n += 3 * d + i + 2 + m.q_rank * (d + 1) + m.heads * (m.dim + m.rot_dim) * m.q_rank
+            n += m.heads * (m.dim + m.vdim) * m.kv_rank + d * m.heads * m.vdim
+            if m.kv_from is None:
+                n += (m.kv_rank + m.rot_dim) * d + m.kv_rank
+            if isinstance(layer.mlp, GluSpec):
+                n += 3 * d * layer.mlp.ff
+            elif isinstance(layer.mlp, MoeSpec):
+                n += layer.mlp.experts * (3 * d * layer.mlp.expert.ff + d)
+                n += 3 * d * layer.mlp.shared.ff if layer.mlp.shared else 0
+        return n
+
+    def kv_bytes_per_token(self, dtype_bytes: int = 2) -> int:
+        return sum((self.layers[i].mixer.kv_rank + self.layers[i].mixer.rot_dim) for i in self.cache_layers()) * dtype_bytes
+
+    def state_bytes_per_seq(self) -> int:
+        return self.num_layers * self.hidden_size * 4
+
+    def replace(self, **kw) -> "BozevikConfig":
+        return dataclasses.replace(self, **kw)
+
+
+def _glu(d: dict) -> GluSpec:
+    return GluSpec(ff=int(d["ff"]), limit=float(d["limit"]))
+
+
+def bozevik_from_config(cfg: dict, name: str = "bozevik") -> BozevikConfig:
+    """A Bozevik checkpoint's config.json: every size and constant is read here; a key this reader does not
+    know means a mechanism this code does not have, so it raises rather than ignore it."""
+    layers = []
+    for i, L in enumerate(cfg["layers"]):
+        if L["type"] != "latent_attention":
+            raise ValueError(f"layer {i}: unknown mixer type {L['type']!r}")
+        m = dict(L["mixer"])
+        rot = dict(m.pop("rot"))
+        spec = LatentMixerSpec(heads=int(m.pop("heads")), dim=int(m.pop("dim")), rot_dim=int(m.pop("rot_dim")),
+                               vdim=int(m.pop("vdim")), kv_rank=int(m.pop("kv_rank")), q_rank=int(m.pop("q_rank")),
+                               rot_base=float(rot.pop("base")), rot_dims=int(rot.pop("dims")), scale=float(m.pop("scale")),
+                               kv_from=(lambda v: None if v is None else int(v))(m.pop("kv_from", None)))
+        if m or rot:
+            raise ValueError(f"layer {i}: unknown mixer keys {sorted(m) + sorted(rot)}")
+        if spec.rot_dims > spec.rot_dim or spec.rot_dims % 2:
+            raise ValueError(f"layer {i}: rot.dims {spec.rot_dims} must be even and <= rot_dim {spec.rot_dim}")
+        if spec.kv_from is not None:
+            src = layers[spec.kv_from].mixer if 0 <= spec.kv_from < i else None
+            if src is None or src.kv_from is not None or (src.kv_rank, src.rot_dim, src.rot_base, src.rot_dims) != (
+                    spec.kv_rank, spec.rot_dim, spec.rot_base, spec.rot_dims):
+                raise ValueError(f"layer {i}: kv_from {spec.kv_from} must name an earlier layer that owns a cache of "
+                                 "the same latent / rotary sizes")
+        mlp = L.get("mlp")
+        if mlp is None:
+            ff = None
+        elif mlp["kind"] == "dense":
+            ff = _glu(mlp)
+        elif mlp["kind"] == "moe":
+            ff = MoeSpec(experts=int(mlp["router"]["experts"]), top=int(mlp["router"]["top"]), expert=_glu(mlp["expert"]),
+                         shared=_glu(mlp["shared"]) if mlp.get("shared") else None)
+        else:
+            raise ValueError(f"layer {i}: unknown mlp kind {mlp['kind']!r}")
+        layers.append(LayerSpec(type=L["type"], mixer=spec, mlp=ff))
+    return BozevikConfig(name=name, vocab_size=int(cfg["vocab"]), hidden_size=int(cfg["width"]), layers=tuple(layers),
+                         norm_eps=float(cfg["norm"]["eps"]), logit_scale=float(cfg.get("logit_scale", 1.0)),
+                         bos_token_id=int(cfg.get("bos_token_id", 1)),
+                         eos_token_ids=tuple(cfg.get("eos_token_ids", (2,))))
+
+
+def bozevik_to_config(c: BozevikConfig) -> dict:
+    """The config.json form of a BozevikConfig (exports, tests)."""
+    layers = []
+    for layer in c.layers:
+        m = layer.mixer
+        md = {"dim": m.dim, "heads": m.heads, "kv_rank": m.kv_rank, "q_rank": m.q_rank,
+              "rot": {"base": m.rot_base, "dims": m.rot_dims}, "rot_dim": m.rot_dim, "scale": m.scale, "vdim": m.vdim}
+        if m.kv_from is not None:
+            md["kv_from"] = m.kv_from
+        f = layer.mlp
+        if f is None:
+            fd = None
+        elif isinstance(f, GluSpec):
+            fd = {"ff": f.ff, "kind": "dense", "limit": f.limit}
+        else:
+            fd = {"expert": {"ff": f.expert.ff, "limit": f.expert.limit}, "kind": "moe",
+                  "router": {"experts": f.experts, "top": f.top}}
+            if f.shared:
+                fd["shared"] = {"ff": f.shared.ff, "limit": f.shared.limit}
+        layers.append({"mixer": md, "mlp": fd, "type": layer.type})
+    return {"architecture": "Bozevik", "layers": layers, "logit_scale": c.logit_scale, "norm": {"eps": c.norm_eps},
+            "vocab": c.vocab_size, "width": c.hidden_size}
+
+
+def _bozevik_stack(name, vocab, width, n_layers, heads, dim, rot_dim, vdim, kv_rank, q_rank, ff, experts=0, top=2,
+                   expert_ff=0, shared_ff=0, share_every=2, **kw) -> BozevikConfig:
+    """n_layers latent-attention layers; every ``share_every``-th attends the previous owner's cache; with experts > 0
+    those layers route (the others are dense)."""
+    layers, owner = [], 0
+    for i in range(n_layers):
+        shares = share_every > 0 and i % share_every == share_every - 1
+        if not shares:
+            owner = i
+        mix = LatentMixerSpec(heads, dim, rot_dim, vdim, kv_rank, q_rank, 10000.0, rot_dim, (dim + rot_dim) ** -0.5,
+                              owner if shares else None)
+        if experts and shares:
+            mlp = MoeSpec(experts, top, GluSpec(expert_ff, 7.0), GluSpec(shared_ff, 7.0) if shared_ff else None)
+        else:
+            mlp = GluSpec(ff, 7.0)
+        layers.append(LayerSpec("latent_attention", mix, mlp))
+    return BozevikConfig(name=name, vocab_size=vocab, hidden_size=width, layers=tuple(layers), **kw)
+
+
+TINY_BOZEVIK = _bozevik_stack("tiny-bozevik", 512, 128, 4, heads=4, dim=16, rot_dim=16, vdim=16, kv_rank=64, q_rank=48,
+                              ff=256, experts=4, top=2, expert_ff=64, shared_ff=64, max_position=2048, bos_token_id=500,
+                              eos_token_ids=(501, 502))
+# layer shapes of a mid-size latent-attention model (benchmarks; random weights)
+SMALL_BOZEVIK = _bozevik_stack("small-bozevik", 32768, 2048, 4, heads=16, dim=128, rot_dim=64, vdim=128, kv_rank=512,
+                               q_rank=1536, ff=8192, share_every=0, max_position=8192, bos_token_id=32000,
+                               eos_token_ids=(32001, 32002))
+SMALL_BOZEVIK_MOE = _bozevik_stack("small-bozevik-moe", 32768, 2048, 4, heads=16, dim=128, rot_dim=64, vdim=128,
+                                   kv_rank=512, q_rank=1536, ff=8192, experts=16, top=4, expert_ff=1024, shared_ff=2048,
+                                   max_position=8192, bos_token_id=32000, eos_token_ids=(32001, 32002))
+
 LLAMA31_SCALING = {
     "rope_type": "llama3",
     "factor": 8.0,
@@ -102,7 +295,7 @@ SMALL_LLAMA = ModelConfig(
 _REGISTRY = {
     c.name: c
     for c in (LLAMA3_8B, LLAMA31_8B, LLAMA3_70B, LLAMA31_70B, MIXTRAL_8X7B, TINY_LLAMA, TINY_MIXTRAL, SMALL_LLAMA,
-              TINY_LLAMA_KV8, TINY_MIXTRAL_E8)
+              TINY_LLAMA_KV8, TINY_MIXTRAL_E8, TINY_BOZEVIK, SMALL_BOZEVIK, SMALL_BOZEVIK_MOE)
 }
 _ALIASES = {
     "llama3": "llama3:8b",
@@ -131,6 +324,14 @@ def resolve(model_name: str) -> ModelConfig:
 
 def known_models() -> list[str]:
     return sorted(set(_REGISTRY) | set(_ALIASES))
+
+
+def from_config_json(cfg: dict, name: str = "hf"):
+    """The model configuration of a checkpoint directory's config.json: the design is chosen by its
+    ``architecture`` key (Bozevik), otherwise the HuggingFace Llama / Mixtral keys."""
+    if cfg.get("architecture") == "Bozevik":
+        return bozevik_from_config(cfg, name)
+    return from_hf_config(cfg, name)
 
 
 def from_hf_config(cfg: dict, name: str = "hf") -> ModelConfig:

@@ -113,6 +113,13 @@ class ForwardBatch:
     top_k: torch.Tensor | None = None       # [num_seqs] int32 (0 = off)
     top_p: torch.Tensor | None = None       # [num_seqs] f32 (1 = off)
     filtered: bool = False                  # some row needs the top-k / top-p resampler
+    sample: bool = True                     # False: no sequence keeps this step's sample (the model may skip sampling)
+    logit_rows: torch.Tensor | None = None  # [n] int64 token rows whose fp32 logits the caller wants (model.last_logits)
+    # models with per-sequence carried state (has_seq_state)
+    prev_row: torch.Tensor | None = None    # [T] int32: >= 0 previous token's row in this step; -1 none (position 0);
+                                            #            <= -2: the sequence's state slot -(v + 2)
+    save_slot: torch.Tensor | None = None   # [T] int32: state slot a sequence's last row of this step is saved to, or -1
+    row_seq: torch.Tensor | None = None     # [T] int32: batch index (block-table row) of each token row
 
     @property
     def num_tokens(self) -> int:
@@ -303,6 +310,11 @@ class TransformerLM:
             ks.append(self.w.layer(0, "w_gu").shape[0] // 2)
         return (self.D == 128 and all(k % 256 == 0 for k in ks) and cfg.hidden_size % 16 == 0
                 and self.vocab_shard % 16 == 0)
+
+    has_seq_state = False  # no per-sequence state besides the paged KV cache
+
+    def make_cache(self, num_blocks: int, block_size: int, num_slots: int = 0) -> KVCache:
+        return KVCache(self.cfg.num_layers, num_blocks, self.hkv, self.D, block_size, self.device)
 
     # ------------------------------------------------------------------------------------------
     def _buf(self, name, shape, dtype):

@@ -178,6 +178,8 @@ def shard_shape(cfg: ModelConfig, shard: ShardSpec, name: str, shape: tuple) -> 
 def random_weights(cfg: ModelConfig, shard: ShardSpec | None = None, device="cpu", dtype=torch.bfloat16,
                    seed: int = 0, mode: str = "full") -> ModelWeights:
     shard = shard or ShardSpec()
+    if getattr(cfg, "family", "llama") == "bozevik":
+        return bozevik_random_weights(cfg, shard, device, dtype, seed)
     shard.validate(cfg)
     shapes = full_shapes(cfg)
     tensors = {}
@@ -230,6 +232,8 @@ def load_hf_weights(path: str, cfg: ModelConfig, shard: ShardSpec | None = None,
     from safetensors import safe_open
 
     shard = shard or ShardSpec()
+    if getattr(cfg, "family", "llama") == "bozevik":
+        return load_bozevik_weights(path, cfg, shard, device, dtype)
     shard.validate(cfg)
     wmap = _hf_index(path)
     handles = {}
@@ -294,3 +298,103 @@ def save_hf_weights(weights: ModelWeights, path: str) -> None:
             out[h + "mlp.down_proj.weight"] = t[p + "w_down"]
     os.makedirs(path, exist_ok=True)
     save_file({k: v.contiguous().cpu() for k, v in out.items()}, os.path.join(path, "model.safetensors"))
+
+
+# --------------------------------------------------------------------------------------------------
+# Bozevik checkpoints: tensors keep the checkpoint's names (embed, l<i>.norm1, l<i>.mix.dq, l<i>.mlp.e<j>.gate, ...);
+# the model fuses what its GEMMs read (models/bozevik.py).  Linear weights are [out, in].
+# --------------------------------------------------------------------------------------------------
+def bozevik_shapes(cfg) -> dict:
+    from .config import GluSpec, MoeSpec
+
+    d = cfg.hidden_size
+    shapes = {"embed": (cfg.vocab_size, d), "final.norm": (d,)}
+    for i, layer in enumerate(cfg.layers):
+        p, m = f"l{i}.", layer.mixer
+        shapes[p + "norm1"] = (d,)
+        shapes[p + "norm2"] = (d,)
+        shapes[p + "shift"] = (d,)
+        shapes[p + "dwa"] = (i + 2,)
+        shapes[p + "mix.dq"] = (m.q_rank, d)
+        shapes[p + "mix.dq.norm"] = (m.q_rank,)
+        shapes[p + "mix.uq"] = (m.heads * (m.dim + m.rot_dim), m.q_rank)
+        if m.kv_from is None:
+            shapes[p + "mix.dkv"] = (m.kv_rank + m.rot_dim, d)
+            shapes[p + "mix.dkv.norm"] = (m.kv_rank,)
+        shapes[p + "mix.uk"] = (m.heads * m.dim, m.kv_rank)
+        shapes[p + "mix.uv"] = (m.heads * m.vdim, m.kv_rank)
+        shapes[p + "mix.o"] = (d, m.heads * m.vdim)
+
+        def glu(prefix, f):
+            shapes[prefix + "gate"], shapes[prefix + "up"], shapes[prefix + "down"] = (f, d), (f, d), (d, f)
+
+        if isinstance(layer.mlp, GluSpec):
+            glu(p + "mlp.", layer.mlp.ff)
+        elif isinstance(layer.mlp, MoeSpec):
+            for e in range(layer.mlp.experts):
+                glu(f"{p}mlp.e{e}.", layer.mlp.expert.ff)
+            shapes[p + "mlp.router"] = (layer.mlp.experts, d)
+            if layer.mlp.shared:
+                glu(p + "mlp.shared.", layer.mlp.shared.ff)
+    return shapes
+
+
+def bozevik_random_weights(cfg, shard: ShardSpec | None = None, device="cpu", dtype=torch.bfloat16,
+                           seed: int = 0) -> ModelWeights:
+    """Random init (benchmarks, tests): matrices N(0, (1.28 / sqrt(fan_in))^2), norm weights 1, token-shift weights
+    uniform in [0, 1), depth weights uniform with the newest layer's raised (a plain residual stream plus a tail)."""
+    shard = shard or ShardSpec()
+    if shard.tp_size > 1 or shard.ep_size > 1:
+        raise NotImplementedError("Bozevik runs on one GPU per replica (its tensors are not sharded)")
+    tensors = {}
+    for name, shape in bozevik_shapes(cfg).items():
+        sd = _seed(seed, name)
+        if name.endswith("shift") or name.endswith("dwa"):
+            g = torch.Generator().manual_seed(sd)
+            t = torch.rand(shape, generator=g)
+            if name.endswith("dwa"):
+                t = t * (0.5 / len(t))
+                t[-1] += 1.0
+            tensors[name] = t.to(dtype).to(device)
+        elif len(shape) == 1:
+            tensors[name] = torch.ones(shape, dtype=dtype, device=device)
+        else:
+            tensors[name] = _randn(shape, sd, device, dtype, 1.0 if name == "embed" else _std(name, shape))
+    return ModelWeights(cfg, shard, tensors)
+
+
+def load_bozevik_weights(path: str, cfg, shard: ShardSpec | None = None, device="cpu",
+                         dtype=torch.bfloat16) -> ModelWeights:
+    """model.safetensors of a Bozevik checkpoint directory; every tensor the configuration implies must be there
+    with the implied shape, and no other."""
+    from safetensors import safe_open
+
+    shard = shard or ShardSpec()
+    if shard.tp_size > 1 or shard.ep_size > 1:
+        raise NotImplementedError("Bozevik runs on one GPU per replica (its tensors are not sharded)")
+    shapes = bozevik_shapes(cfg)
+    tensors = {}
+    with safe_open(os.path.join(path, "model.safetensors"), framework="pt") as f:
+        names = set(f.keys())
+        missing, extra = sorted(set(shapes) - names), sorted(names - set(shapes))
+        if missing or extra:
+            raise ValueError(f"checkpoint does not fit its config: missing {missing[:4]}, unexpected {extra[:4]}")
+        for name, shape in shapes.items():
+            t = f.get_tensor(name)
+            if tuple(t.shape) != tuple(shape):
+                raise ValueError(f"{name}: shape {tuple(t.shape)}, the config implies {tuple(shape)}")
+            tensors[name] = t.to(dtype).to(device)
+    return ModelWeights(cfg, shard, tensors)
+
+
+def save_bozevik_checkpoint(weights: ModelWeights, path: str) -> None:
+    """config.json + model.safetensors (bf16) of a Bozevik model, in the form the loader reads."""
+    from safetensors.torch import save_file
+
+    from .config import bozevik_to_config
+
+    os.makedirs(path, exist_ok=True)
+    with open(os.path.join(path, "config.json"), "w") as f:
+        json.dump(bozevik_to_config(weights.cfg), f, indent=1)
+    save_file({k: v.detach().to(torch.bfloat16).contiguous().cpu() for k, v in weights.tensors.items()},
+              os.path.join(path, "model.safetensors"))

@@ -576,3 +576,119 @@ def choose_splits(N: int, K: int, target_wgs: int = 1024, min_k_per_wave: int = 
         if tiles * s >= target_wgs:
             break
     return best
+
+
+# ======================================================================================================
+# Mechanisms of the latent-attention model family (csrc/kernels/seq_mix.hip, latent_attention.hip, glu_moe.hip):
+# activations bf16 or fp32 (a model served in 32-bit), residual stream / carried state / statistics / scores fp32.
+# ======================================================================================================
+def _lat():
+    return _native.latent_ops()
+
+
+def embed_rows(ids, table, x, hist0, src=None, prev=None):
+    """x = hist0 = table[token] (fp32); rows with src >= 0 take the token prev[src] (previous step's device sample)."""
+    if _gpu(x):
+        return _lat().embed_rows(ids, src, prev, table, x, hist0)
+    return reference.embed_rows(reference.resolve_ids(ids, src, prev), table, x, hist0)
+
+
+def token_shift(x, mu, prev_row, state, h):
+    """h = x + (x_prev - x) * mu.  prev_row[r] >= 0: row of x; -1: zeros (first token); <= -2: state[-(v + 2)]
+    (the sequence's carried row: the layer input of its last token of an earlier step); state [slots, d] fp32."""
+    if _gpu(x):
+        return _lat().token_shift(x, mu, prev_row, state, h)
+    return reference.token_shift(x, mu, prev_row, state, h)
+
+
+def add_layer_norm(delta, w, eps, x, save=None, state=None, hist=None, coef=None, hist_idx=0, out_act=None):
+    """x += layer_norm(delta) * w (weight, no bias; variance = mean of squared deviations).  Optional:
+    ``save``/``state``: rows with save[r] >= 0 first store the OLD x row into state[save[r]] (the carried state of
+    the next step's token shift); ``hist``/``coef``/``hist_idx``: hist[hist_idx] = x_new, then
+    x = sum_j coef[j] * hist[j] over j <= hist_idx (depth-weighted average of the layer outputs);
+    ``out_act``: the result in the activation dtype."""
+    if _gpu(x):
+        return _lat().add_layer_norm(delta, w, float(eps), x, save, state, hist, coef, int(hist_idx), out_act)
+    return reference.add_layer_norm(delta, w, eps, x, save, state, hist, coef, hist_idx, out_act)
+
+
+def layer_norm(x, rows, w, eps, out):
+    """out[i] = layer_norm(x[rows[i]]) * w (rows None: the first len(out) rows)."""
+    if _gpu(x):
+        return _lat().layer_norm(x, rows, w, float(eps), out)
+    return reference.layer_norm(x, rows, w, eps, out)
+
+
+def rope_pair_table(max_pos: int, dims: int, base: float, device=None) -> torch.Tensor:
+    """[max_pos, dims / 2, 2] fp32 (cos, sin) of the angles p * base^(-2i / dims), for the interleaved-pair rotary."""
+    return reference.rope_pair_table(max_pos, dims, base, device)
+
+
+def latent_prep(z, q_rank, kv_rank, rot, wq, wkv, eps, positions, slots, rope, cq, cache):
+    """z [T, q_rank (+ kv_rank + rot)] -> cq = rms_norm(z[:, :q_rank]) * wq; with a kv part (kv_rank > 0) the token's
+    cache row (slot >= 0) becomes [rms_norm(z kv part) * wkv | rotary(z rot part)]."""
+    if _gpu(z):
+        return _lat().latent_prep(z, int(q_rank), int(kv_rank), int(rot), wq, wkv, float(eps), positions, slots, rope,
+                                  cq, cache)
+    return reference.latent_prep(z, q_rank, kv_rank, rot, wq, wkv, eps, positions, slots, rope, cq, cache)
+
+
+def rope_pairs(src, dst, positions, rope):
+    """Interleaved-pair rotary of a [T, H, rot] view into another (unit inner strides)."""
+    if _gpu(src):
+        return _lat().rope_pairs(src, dst, positions, rope)
+    return reference.rope_pairs(src, dst, positions, rope)
+
+
+LATENT_ATTN_PART = 256  # keys per split-KV partition of latent_attn's decode form (latent_attention.hip PART)
+
+
+def latent_attn(q, cache, block_tables, row_seq, positions, scale, kv_rank, out, part_o=None, part_ml=None):
+    """Causal softmax attention of q [T, H, Dk] over the paged latent cache [NB, BS, Dk]: keys are whole cache rows,
+    values their first kv_rank entries; row r sees keys 0..positions[r] of sequence row_seq[r].  ``part_o`` /
+    ``part_ml``: split-KV scratch (decode steps: one partition per 256 keys, merged in a second launch)."""
+    if _gpu(q):
+        return _lat().latent_attn(q, cache, block_tables, row_seq, positions, float(scale), int(kv_rank), out, part_o,
+                                  part_ml)
+    return reference.latent_attn(q, cache, block_tables, row_seq, positions, scale, kv_rank, out)
+
+
+def clamped_glu(gu, limit, alpha, out):
+    """gu [R, 2F] = gate | up -> out = g * sigmoid(alpha * g) * (u + 1), g = min(gate, limit), u = clamp(up, +-limit)."""
+    if _gpu(gu):
+        return _lat().clamped_glu(gu, float(limit), float(alpha), out)
+    return reference.clamped_glu(gu, limit, alpha, out)
+
+
+def sigmoid_topk(x, Wr, k, ids, w):
+    """Router: fp32 scores sigmoid(x @ Wr.T); the k largest per row -> ids [T, k] int32, w [T, k] fp32 (the scores)."""
+    if _gpu(x):
+        return _lat().sigmoid_topk(x, Wr, int(k), ids, w)
+    return reference.sigmoid_topk(x, Wr, k, ids, w)
+
+
+def expert_offsets(ids, R, E, offsets, cursor):
+    if _gpu(ids):
+        return _lat().expert_offsets(ids, int(R), int(E), offsets, cursor)
+    return reference.expert_offsets(ids, R, E, offsets, cursor)
+
+
+def scatter_scaled(x, ids, w, k, offsets, cursor, xs, dst):
+    """xs[dst[a]] = w[a] * x[a // k] with the rows of expert e in [offsets[e], offsets[e + 1])."""
+    if _gpu(x):
+        return _lat().scatter_scaled(x, ids, w, int(k), offsets, cursor, xs, dst)
+    return reference.scatter_scaled(x, ids, w, k, offsets, cursor, xs, dst)
+
+
+def grouped_linear(xs, W, offsets, y):
+    """y[r] = xs[r] @ W[e].T for the rows of expert e's segment; any shape, bf16 or fp32."""
+    if _gpu(xs):
+        return _lat().grouped_linear(xs, W, offsets, y)
+    return reference.grouped_linear(xs, W, offsets, y)
+
+
+def gather_sum(y, dst, k, extra, out):
+    """out[t] = sum_j y[dst[t * k + j]] (+ extra[t]) in fp32."""
+    if _gpu(out):
+        return _lat().gather_sum(y, dst, int(k), extra, out)
+    return reference.gather_sum(y, dst, k, extra, out)

@@ -53,3 +53,27 @@ def ops():
 
 def library_path() -> str:
     return _LIB
+
+
+# ---- the latent-attention / carried-state / clamped-GLU kernels: symmetry_amd/_C_latent.so ------------------------
+_LATENT_LIB = os.path.join(os.path.dirname(_LIB), "_C_latent.so")
+_latent_loaded = False
+
+
+def latent_ops():
+    """``torch.ops.symmetry_amd_latent`` (loaded once; built first if the library is missing: three translation
+    units, about half a minute).  Raises if it cannot be built or loaded: no eager fallback on the device."""
+    global _latent_loaded
+    with _lock:
+        if not _latent_loaded:
+            if not os.path.exists(_LATENT_LIB):
+                from symmetry_amd import _build
+
+                _build.build_latent()
+            torch.ops.load_library(_LATENT_LIB)
+            _latent_loaded = True
+    return torch.ops.symmetry_amd_latent
+
+
+def latent_library_path() -> str:
+    return _LATENT_LIB

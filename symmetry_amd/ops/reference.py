@@ -553,3 +553,149 @@ def moe_combine_prep(y, dst, ids, E: int, w, k: int, resid, w_next, xw, ss) -> N
     out = torch.empty(T, d, dtype=torch.float32)
     moe_combine(y, dst, ids, 0, E, w, k, out, False)
     add_prep(out, resid, w_next, xw, ss)
+
+
+# ======================================================================================================
+# torch references of the latent-attention model family's ops (CPU path of symmetry_amd.ops; same contracts:
+# outputs written in place, activations in the tensors' own dtype, statistics / scores / sums in fp32)
+# ======================================================================================================
+def embed_rows(ids, table, x, hist0) -> None:
+    v = table[ids.long()].float()
+    x.copy_(v)
+    hist0.view_as(x).copy_(v)
+
+
+def token_shift(x, mu, prev_row, state, h) -> None:
+    T = x.shape[0]
+    pr = prev_row[:T].long()
+    prev = torch.zeros_like(x)
+    rows = pr >= 0
+    prev[rows] = x[pr[rows]]
+    st = pr <= -2
+    prev[st] = state[-(pr[st] + 2)]
+    h.copy_((x + (prev - x) * mu.float()).to(h.dtype))
+
+
+def _ln(v, w, eps):
+    mean = v.mean(-1, keepdim=True)
+    var = ((v - mean) ** 2).mean(-1, keepdim=True)
+    return (v - mean) / torch.sqrt(var + eps) * w.float()
+
+
+def add_layer_norm(delta, w, eps, x, save, state, hist, coef, hist_idx, out_act) -> None:
+    T = x.shape[0]
+    if save is not None:
+        sv = save[:T].long()
+        keep = sv >= 0
+        state[sv[keep]] = x[keep]
+    xn = x + _ln(delta.float().view_as(x), w, eps)
+    if hist is not None:
+        hist[hist_idx].copy_(xn)
+        xn = (coef.float().view(-1, 1, 1) * hist[: hist_idx + 1]).sum(0)
+    x.copy_(xn)
+    if out_act is not None:
+        out_act.copy_(xn.to(out_act.dtype))
+
+
+def layer_norm(x, rows, w, eps, out) -> None:
+    n = out.shape[0]
+    v = x[rows[:n].long()] if rows is not None else x[:n]
+    out.copy_(_ln(v, w, eps).to(out.dtype))
+
+
+def rope_pair_table(max_pos: int, dims: int, base: float, device=None) -> torch.Tensor:
+    i = torch.arange(dims // 2, dtype=torch.float64)
+    freq = (torch.tensor(float(base), dtype=torch.float64) ** (-2.0 * i / dims)).float()  # angles are fp32 products
+    a = torch.arange(max_pos, dtype=torch.float32)[:, None] * freq[None, :]
+    a = a.double()
+    return torch.stack([torch.cos(a), torch.sin(a)], -1).float().to(device or "cpu")
+
+
+def _rot_pairs(v, cs):
+    """v [..., rot] fp32, cs [..., rot/2, 2] broadcastable."""
+    u, w = v[..., 0::2], v[..., 1::2]
+    c, s = cs[..., 0], cs[..., 1]
+    return torch.stack([u * c - w * s, w * c + u * s], -1).flatten(-2)
+
+
+def latent_prep(z, q_rank, kv_rank, rot, wq, wkv, eps, positions, slots, rope, cq, cache) -> None:
+    T = z.shape[0]
+    zf = z.float()
+    q = zf[:, :q_rank]
+    cq.copy_((q / torch.sqrt((q * q).mean(-1, keepdim=True) + eps) * wq.float()).to(cq.dtype))
+    if not kv_rank:
+        return
+    c = zf[:, q_rank:q_rank + kv_rank]
+    c = c / torch.sqrt((c * c).mean(-1, keepdim=True) + eps) * wkv.float()
+    kr = _rot_pairs(zf[:, q_rank + kv_rank:], rope[positions[:T].long()])
+    row = torch.cat([c, kr], -1).to(cache.dtype)
+    sl = slots[:T].long()
+    keep = sl >= 0
+    cache.view(-1, kv_rank + rot)[sl[keep]] = row[keep]
+
+
+def rope_pairs(src, dst, positions, rope) -> None:
+    T = src.shape[0]
+    dst.copy_(_rot_pairs(src.float(), rope[positions[:T].long()][:, None]).to(dst.dtype))
+
+
+def latent_attn(q, cache, block_tables, row_seq, positions, scale, kv_rank, out) -> None:
+    T, H, Dk = q.shape
+    BS = cache.shape[1]
+    o = out.view(T, H, kv_rank)
+    for r in range(T):
+        n = int(positions[r]) + 1
+        bt = block_tables[int(row_seq[r])].long()
+        idx = torch.arange(n)
+        rows = cache[bt[idx // BS], idx % BS].float()          # [n, Dk]
+        s = (q[r].float() @ rows.t()) * scale                   # [H, n]
+        p = torch.softmax(s, -1)
+        o[r] = (p @ rows[:, :kv_rank]).to(out.dtype)
+
+
+def clamped_glu(gu, limit, alpha, out) -> None:
+    F = out.shape[1]
+    g = gu[:, :F].float().clamp(max=limit)
+    u = gu[:, F:].float().clamp(-limit, limit)
+    out.copy_((g * torch.sigmoid(alpha * g) * (u + 1)).to(out.dtype))
+
+
+def sigmoid_topk(x, Wr, k, ids, w) -> None:
+    T = x.shape[0]
+    s = torch.sigmoid(x.float() @ Wr.float().t())
+    top = s.topk(k, dim=-1)
+    ids[: T * k].copy_(top.indices.reshape(-1).int())
+    w[: T * k].copy_(top.values.reshape(-1))
+
+
+def expert_offsets(ids, R, E, offsets, cursor) -> None:
+    counts = torch.bincount(ids[:R].long(), minlength=E)
+    offsets[0] = 0
+    offsets[1:E + 1] = counts.cumsum(0).int()
+    cursor[:E] = 0
+
+
+def scatter_scaled(x, ids, w, k, offsets, cursor, xs, dst) -> None:
+    R = x.shape[0] * k
+    e = ids[:R].long()
+    order = torch.sort(e, stable=True).indices       # assignment a lands at the rank of (expert, a)
+    pos = torch.empty(R, dtype=torch.long)
+    pos[order] = torch.arange(R)
+    dst[:R] = pos.int()
+    xs.view(R, -1)[pos] = (w[:R, None] * x.float().repeat_interleave(k, 0)).to(xs.dtype)
+
+
+def grouped_linear(xs, W, offsets, y) -> None:
+    offs = offsets.tolist()
+    for e in range(W.shape[0]):
+        a, b = offs[e], offs[e + 1]
+        if b > a:
+            y[a:b] = (xs[a:b].float() @ W[e].float().t()).to(y.dtype)
+
+
+def gather_sum(y, dst, k, extra, out) -> None:
+    T = out.shape[0]
+    s = y.float()[dst[: T * k].long()].view(T, k, -1).sum(1)
+    if extra is not None:
+        s = s + extra.float().view_as(s)
+    out.copy_(s)
