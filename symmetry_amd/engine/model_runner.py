@@ -442,7 +442,7 @@ class ModelRunner:
             lg = handle.pop("logits")
             pick = handle.pop("logit_pick")
             lg = lg if pick is None else lg[torch.as_tensor(pick, device=lg.device)]
-            handle["logits_host"] = lg.float().cpu()
+            handle["logits_host"] = lg.to("cpu", torch.float32, copy=True)  # (a copy also on the CPU: workspace memory)
         return ids[:handle["nseq"]]
 
     @staticmethod
