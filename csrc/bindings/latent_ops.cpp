@@ -185,9 +185,9 @@ void rope_pairs(const Tensor& src, Tensor& dst, const Tensor& positions, const T
                     ptr<int>(positions), ptr<float>(rope), (int)T, (int)H, (int)rot, f32, cur_stream(src));
 }
 
-void latent_attn(const Tensor& q, const Tensor& cache, const Tensor& block_tables, const Tensor& row_seq,
-                 const Tensor& positions, double scale, int64_t kv_rank, Tensor& out, const OptTensor& part_o,
-                 const OptTensor& part_ml) {
+int64_t latent_attn(const Tensor& q, const Tensor& cache, const Tensor& block_tables, const Tensor& row_seq,
+                    const Tensor& positions, double scale, int64_t kv_rank, Tensor& out, const OptTensor& part_o,
+                    const OptTensor& part_ml, const OptTensor& tiles, const OptTensor& cu_q, int64_t impl) {
   const int f32 = act(q, "q");
   same_act(cache, f32, "cache");
   same_act(out, f32, "out");
@@ -224,7 +224,20 @@ void latent_attn(const Tensor& q, const Tensor& cache, const Tensor& block_table
   a.positions = ptr<int>(positions);
   a.out = out.data_ptr();
   a.scale = (float)scale;
-  launch_latent_attn(a, f32, cur_stream(q));
+  if (tiles.has_value()) {
+    TORCH_CHECK(cu_q.has_value() && !part_o.has_value(), "latent_attn: tiles need cu_q and take no split-KV partials");
+    dtype(*tiles, at::kInt, "tiles");
+    dtype(*cu_q, at::kInt, "cu_q");
+    TORCH_CHECK(tiles->dim() == 2 && tiles->size(1) == 2 && cu_q->numel() == block_tables.size(0) + 1,
+                "latent_attn: tiles [n, 2], cu_q [seqs + 1]");
+    a.tiles = ptr<int>(*tiles);
+    a.cu_q = ptr<int>(*cu_q);
+    a.ntiles = (int)tiles->size(0);
+  }
+  TORCH_CHECK(q.data_ptr() != nullptr && (reinterpret_cast<uintptr_t>(q.data_ptr()) % 16 == 0) &&
+                  (reinterpret_cast<uintptr_t>(cache.data_ptr()) % 16 == 0) &&
+                  (reinterpret_cast<uintptr_t>(out.data_ptr()) % 16 == 0), "latent_attn: 16-byte aligned tensors");
+  return launch_latent_attn(a, f32, (int)impl, cur_stream(q));
 }
 
 int64_t latent_attn_part() { return latent_attn_part_tokens(); }
@@ -319,7 +332,7 @@ TORCH_LIBRARY(symmetry_amd_latent, m) {
   m.def("rope_pairs(Tensor src, Tensor(a!) dst, Tensor positions, Tensor rope) -> ()", &rope_pairs);
   m.def(
       "latent_attn(Tensor q, Tensor cache, Tensor block_tables, Tensor row_seq, Tensor positions, float scale, "
-      "int kv_rank, Tensor(a!) out, Tensor(b!)? part_o, Tensor(c!)? part_ml) -> ()",
+      "int kv_rank, Tensor(a!) out, Tensor(b!)? part_o, Tensor(c!)? part_ml, Tensor? tiles, Tensor? cu_q, int impl) -> int",
       &latent_attn);
   m.def("latent_attn_part() -> int", &latent_attn_part);
   m.def("clamped_glu(Tensor gu, float limit, float alpha, Tensor(a!) out) -> ()", &clamped_glu);

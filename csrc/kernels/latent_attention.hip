@@ -13,7 +13,20 @@
 //   latent_prep   per token: RMS-norm the query latent; RMS-norm the kv latent and rotate the shared key part into
 //                 the token's cache row (statistics and angles in fp32)
 //   rope_pairs    interleaved-pair rotary (dimension 2i with 2i + 1) of a strided [T][H][rot] slice
-//   latent_attn   causal softmax attention over the paged latent cache; scores, weights and accumulators fp32
+//   latent_attn   causal softmax attention over the paged latent cache; scores, weights and accumulators fp32.
+//                 Two implementations: the MFMA kernel (bf16, tiled shapes) and a one-wave-per-(row, head) kernel
+//                 for every other shape and for the 32-bit model.
+//
+// MFMA kernel (v_mfma_f32_16x16x32_bf16, 4 waves, 64 query vectors per workgroup: 64 rows of one head for prompt
+// tiles, one row's heads for decode steps with split-KV partitions).  Per 32-key tile the workgroup stages the cache
+// rows ONCE for all its query vectors -- key-major for the scores, and the latent part a second time transposed
+// (dim-major) for the weighted sum: the score product contracts over the row's dims and the value product over the
+// keys, an MFMA operand wants its contraction index contiguous per lane, and keys and values are the same bytes here,
+// so one transpose per tile is inherent; it happens on the way into LDS, off the HBM / L2 path.  Both products run
+// swapped (S^T = K Q^T, O^T = V^T P^T): the query fragments stay in registers for the whole key loop, the packed
+// bf16 weights of a lane ARE its B operand of the second product (the 32 keys of a tile are consumed in the order
+// the accumulator layout hands them out, and the V^T fragment reads follow the same order), and the softmax
+// statistics of a query vector live in the 4 lanes that share its accumulator column.
 #include "common.h"
 #include "latent_launchers.h"
 
@@ -196,6 +209,181 @@ __global__ __launch_bounds__(64) void latent_attn_merge_kernel(LatentAttnArgs a)
   }
 }
 
+
+constexpr int KT = 32;        // keys per staged tile
+constexpr int LDV = KT + 4;   // row pitch (elements) of the transposed latent tile
+
+template <int NKM, int RTM, bool DECODE>
+__global__ __launch_bounds__(256) void latent_attn_mfma_kernel(LatentAttnArgs a) {
+  extern __shared__ __attribute__((aligned(16))) char smem[];
+  const int Dk = a.Dk, r = a.kv_rank, H = a.H;
+  const int nk = Dk >> 5, rt = r >> 4;
+  const int ldk = Dk + 8;
+  bf16* Ks = reinterpret_cast<bf16*>(smem);  // [KT][ldk] key-major cache rows
+  bf16* Vt = Ks + KT * ldk;                   // [r][LDV] latent part, dim-major
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int n = lane & 15, g = lane >> 4;
+  int seq, qrow, head, limit, k_lo, k_hi, wave_hi, part = 0;
+  bool valid, wave_active;
+  if constexpr (DECODE) {
+    qrow = blockIdx.x;
+    seq = a.row_seq[qrow];
+    head = blockIdx.y * 64 + wave * 16 + n;
+    valid = head < H;
+    wave_active = blockIdx.y * 64 + wave * 16 < H;
+    limit = a.positions[qrow];
+    part = blockIdx.z;
+    k_lo = a.parts > 1 ? part * PART : 0;
+    k_hi = a.parts > 1 ? min(limit + 1, k_lo + PART) : limit + 1;
+    if (k_lo >= k_hi) return;  // a partition past this row's keys: the merge never reads it
+    wave_hi = k_hi;
+  } else {
+    seq = a.tiles[2 * blockIdx.x];
+    const int off = a.tiles[2 * blockIdx.x + 1];
+    const int q0 = a.cu_q[seq], qlen = a.cu_q[seq + 1] - q0;
+    if (off >= qlen) return;  // padding tile
+    const int rin = off + wave * 16 + n;
+    valid = rin < qlen;
+    wave_active = off + wave * 16 < qlen;
+    qrow = q0 + min(rin, qlen - 1);
+    head = blockIdx.y;
+    limit = a.positions[qrow];
+    k_lo = 0;
+    k_hi = a.positions[q0 + min(off + 63, qlen - 1)] + 1;       // a run's rows are consecutive positions
+    wave_hi = a.positions[q0 + min(off + wave * 16 + 15, qlen - 1)] + 1;
+  }
+  const bf16* qp = (const bf16*)a.q + ((long long)qrow * H + min(head, H - 1)) * Dk;
+  bf16x8 qf[NKM];
+#pragma unroll
+  for (int s = 0; s < NKM; ++s)
+    if (s < nk) qf[s] = *reinterpret_cast<const bf16x8*>(qp + s * 32 + g * 8);
+  f32x4 o[RTM];
+#pragma unroll
+  for (int i = 0; i < RTM; ++i) o[i] = f32x4{0.f, 0.f, 0.f, 0.f};
+  float m = -INFINITY, l = 0.f;
+  const int* bt = a.block_tables + (long long)seq * a.max_blocks;
+  const bf16* cache = (const bf16*)a.cache;
+  const int key_in = tid & 31;
+  for (int k0 = k_lo; k0 < k_hi; k0 += KT) {
+    __syncthreads();  // the previous tile's fragment reads are done
+    {
+      const int key = min(k0 + key_in, k_hi - 1);
+      const bf16* src = cache + ((long long)bt[key / a.BS] * a.BS + key % a.BS) * Dk;
+      for (int c = tid >> 5; c < (Dk >> 3); c += 8) {
+        Pack8 pk;
+        pk.u = *reinterpret_cast<const uint4*>(src + c * 8);
+        *reinterpret_cast<uint4*>(Ks + key_in * ldk + c * 8) = pk.u;
+        if (c * 8 < r) {
+#pragma unroll
+          for (int j = 0; j < 8; ++j) Vt[(c * 8 + j) * LDV + key_in] = pk.h[j];
+        }
+      }
+    }
+    __syncthreads();
+    if (!wave_active || k0 >= wave_hi) continue;
+    // S^T: rows = keys (sub * 16 + g * 4 + i), column = this lane's query vector n
+    f32x4 st[2];
+#pragma unroll
+    for (int sub = 0; sub < 2; ++sub) {
+      f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+      const bf16* kr = Ks + (sub * 16 + n) * ldk + g * 8;
+#pragma unroll
+      for (int s = 0; s < NKM; ++s)
+        if (s < nk) acc = mfma16(*reinterpret_cast<const bf16x8*>(kr + s * 32), qf[s], acc);
+      st[sub] = acc;
+    }
+    float mx = -INFINITY;
+#pragma unroll
+    for (int sub = 0; sub < 2; ++sub)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int key = k0 + sub * 16 + g * 4 + i;
+        const float v = (key > limit || key >= k_hi) ? -INFINITY : st[sub][i] * a.scale;
+        st[sub][i] = v;
+        mx = fmaxf(mx, v);
+      }
+    mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+    const float m_new = fmaxf(m, mx);          // finite: every query vector sees the first key of its range
+    const float alpha = __expf(m - m_new);
+    float ps = 0.f;
+    Pack8 pb;
+#pragma unroll
+    for (int sub = 0; sub < 2; ++sub)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const float p = __expf(st[sub][i] - m_new);
+        ps += p;
+        pb.h[sub * 4 + i] = (bf16)p;
+      }
+    ps += __shfl_xor(ps, 16, 64);
+    ps += __shfl_xor(ps, 32, 64);
+    l = l * alpha + ps;
+    m = m_new;
+    // O^T += V^T P^T: k index g * 8 + j of the product is key g * 4 + j (j < 4) / 16 + g * 4 + j - 4 of the tile
+    const bf16* vr = Vt + n * LDV + g * 4;
+#pragma unroll
+    for (int dt = 0; dt < RTM; ++dt)
+      if (dt < rt) {
+        Pack8 va;
+        const uint2 lo = *reinterpret_cast<const uint2*>(vr + dt * 16 * LDV);
+        const uint2 hi = *reinterpret_cast<const uint2*>(vr + dt * 16 * LDV + 16);
+        va.u = make_uint4(lo.x, lo.y, hi.x, hi.y);
+        o[dt] = mfma16(va.v, pb.v, o[dt] * alpha);
+      }
+  }
+  if (!valid) return;
+  // o[dt][i]: dim dt * 16 + g * 4 + i of query vector n
+  if (a.parts == 1) {
+    bf16* out = (bf16*)a.out + ((long long)qrow * H + head) * r;
+    const float inv = 1.f / l;
+#pragma unroll
+    for (int dt = 0; dt < RTM; ++dt)
+      if (dt < rt) {
+        bf16x4 v;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) v[i] = (bf16)(o[dt][i] * inv);
+        *reinterpret_cast<bf16x4*>(out + dt * 16 + g * 4) = v;
+      }
+  } else {
+    const long long pi = ((long long)qrow * H + head) * a.parts + part;
+    float* po = a.part_o + pi * r;
+#pragma unroll
+    for (int dt = 0; dt < RTM; ++dt)
+      if (dt < rt) *reinterpret_cast<f32x4*>(po + dt * 16 + g * 4) = o[dt];
+    if (g == 0) {
+      a.part_ml[2 * pi] = m;
+      a.part_ml[2 * pi + 1] = l;
+    }
+  }
+}
+
+template <int NKM, int RTM>
+void mfma_launch(const LatentAttnArgs& a, hipStream_t s) {
+  const size_t lds = ((size_t)KT * (a.Dk + 8) + (size_t)a.kv_rank * LDV) * sizeof(bf16);
+  static bool raised = false;  // (per instantiation) dynamic LDS beyond the 64 KB default
+  if (!raised) {
+    hipFuncSetAttribute(reinterpret_cast<const void*>(&latent_attn_mfma_kernel<NKM, RTM, true>),
+                        hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024);
+    hipFuncSetAttribute(reinterpret_cast<const void*>(&latent_attn_mfma_kernel<NKM, RTM, false>),
+                        hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024);
+    raised = true;
+  }
+  if (a.tiles)
+    latent_attn_mfma_kernel<NKM, RTM, false><<<dim3(a.ntiles, a.H), 256, lds, s>>>(a);
+  else
+    latent_attn_mfma_kernel<NKM, RTM, true><<<dim3(a.T, (a.H + 63) / 64, a.parts), 256, lds, s>>>(a);
+}
+
+bool mfma_dispatch(const LatentAttnArgs& a, hipStream_t s) {
+  const int nk = a.Dk / 32, rt = a.kv_rank / 16;
+  if (a.Dk % 32 || a.kv_rank % 16 || nk > 18 || rt > 32) return false;
+  if (nk <= 5 && rt <= 8) mfma_launch<5, 8>(a, s);
+  else if (nk <= 10 && rt <= 16) mfma_launch<10, 16>(a, s);
+  else mfma_launch<18, 32>(a, s);
+  return true;
+}
+
 template <typename T>
 void attn_dispatch(const LatentAttnArgs& a, hipStream_t s) {
   dim3 grid(a.T, a.H, a.parts);
@@ -205,7 +393,6 @@ void attn_dispatch(const LatentAttnArgs& a, hipStream_t s) {
   else if (nr <= 2) latent_attn_wave_kernel<T, 2><<<grid, 64, lds, s>>>(a);
   else if (nr <= 4) latent_attn_wave_kernel<T, 4><<<grid, 64, lds, s>>>(a);
   else latent_attn_wave_kernel<T, 8><<<grid, 64, lds, s>>>(a);
-  if (a.parts > 1) latent_attn_merge_kernel<T><<<dim3(a.T, a.H), 64, 0, s>>>(a);
 }
 
 }  // namespace
@@ -227,8 +414,15 @@ void launch_rope_pairs(const void* src, long long s_t, long long s_h, void* dst,
     rope_pairs_kernel<bf16><<<T, NT, 0, s>>>((const bf16*)src, s_t, s_h, (bf16*)dst, d_t, d_h, positions, rope, H, rot);
 }
 
-void launch_latent_attn(const LatentAttnArgs& a, int f32, hipStream_t s) {
-  if (a.T <= 0) return;
-  if (f32) attn_dispatch<float>(a, s);
+int launch_latent_attn(const LatentAttnArgs& a, int f32, int impl, hipStream_t s) {
+  if (a.T <= 0) return 0;
+  int used = 1;
+  if (!f32 && impl == 0 && (a.tiles ? a.ntiles > 0 : true) && mfma_dispatch(a, s)) used = 0;
+  else if (f32) attn_dispatch<float>(a, s);
   else attn_dispatch<bf16>(a, s);
+  if (a.parts > 1) {
+    if (f32) latent_attn_merge_kernel<float><<<dim3(a.T, a.H), 64, 0, s>>>(a);
+    else latent_attn_merge_kernel<bf16><<<dim3(a.T, a.H), 64, 0, s>>>(a);
+  }
+  return used;
 }

@@ -53,8 +53,15 @@ struct LatentAttnArgs {
   float* part_ml;
   int T, H, Dk, kv_rank, BS, max_blocks, parts;
   float scale;
+  // prompt form of the MFMA kernel: 64-row query tiles (sequence, first row within the sequence's run) over the
+  // runs cu_q[seq] .. cu_q[seq + 1]; nullptr: one query row per sequence (decode steps)
+  const int* tiles;
+  const int* cu_q;
+  int ntiles;
 };
-void launch_latent_attn(const LatentAttnArgs& a, int f32, hipStream_t s);
+// impl: 0 = MFMA kernel where the shapes allow (bf16, Dk % 32 == 0, kv_rank % 16 == 0, Dk <= 576, kv_rank <= 512),
+// 1 = always the one-wave-per-(row, head) kernel (all shapes, both dtypes).  Returns the implementation used.
+int launch_latent_attn(const LatentAttnArgs& a, int f32, int impl, hipStream_t s);
 int latent_attn_part_tokens();
 
 // ---- glu_moe.hip -------------------------------------------------------------------------------------

@@ -234,7 +234,7 @@ class LLMEngine:
         return True
 
     def _auto_blocks(self, max_model_len: int) -> int:
-        per_block = self.model_cfg.kv_bytes_per_token(self._kv_elem) // self.cfg.tp_size * self.cfg.block_size
+        per_block = self.model_cfg.kv_bytes_per_token(getattr(self, "_kv_elem", 2)) // self.cfg.tp_size * self.cfg.block_size
         if self.device.type == "cpu":
             want = (self.cfg.max_num_seqs * max_model_len) // self.cfg.block_size + 8
             return max(16, min(want, (1 << 30) // per_block))

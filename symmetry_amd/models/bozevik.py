@@ -209,7 +209,9 @@ class BozevikLM:
             if parts > 1:
                 part_o = self._buf("attn.part_o", (T, H, parts, r), torch.float32)
                 part_ml = self._buf("attn.part_ml", (T, H, parts, 2), torch.float32)
-        ops.latent_attn(qa, plane, b.block_tables, b.row_seq, b.positions, m.scale, r, olat, part_o, part_ml)
+        tiled = b.kind != "decode" and self.dtype == torch.bfloat16
+        ops.latent_attn(qa, plane, b.block_tables, b.row_seq, b.positions, m.scale, r, olat, part_o, part_ml,
+                        b.tiles if tiled else None, b.cu_q if tiled else None)
         ov = self._buf("ov", (T, H * m.vdim))
         torch.bmm(olat.transpose(0, 1), P["uvt"], out=ov.view(T, H, m.vdim).transpose(0, 1))
         return self._linear("att", ov, P["o"])

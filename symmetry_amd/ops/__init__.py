@@ -643,14 +643,23 @@ def rope_pairs(src, dst, positions, rope):
 LATENT_ATTN_PART = 256  # keys per split-KV partition of latent_attn's decode form (latent_attention.hip PART)
 
 
-def latent_attn(q, cache, block_tables, row_seq, positions, scale, kv_rank, out, part_o=None, part_ml=None):
+LATENT_ATTN_IMPL = 1 if os.environ.get("SYMMETRY_LATENT_ATTN", "mfma") == "wave" else 0  # A/B: the all-shapes kernel
+
+
+def latent_attn(q, cache, block_tables, row_seq, positions, scale, kv_rank, out, part_o=None, part_ml=None,
+                tiles=None, cu_q=None, impl=None):
     """Causal softmax attention of q [T, H, Dk] over the paged latent cache [NB, BS, Dk]: keys are whole cache rows,
     values their first kv_rank entries; row r sees keys 0..positions[r] of sequence row_seq[r].  ``part_o`` /
-    ``part_ml``: split-KV scratch (decode steps: one partition per 256 keys, merged in a second launch)."""
+    ``part_ml``: split-KV scratch (decode steps: one partition per 256 keys, merged in a second launch).
+    ``tiles`` [n, 2] (sequence, first row of a 64-row tile within the sequence's run) + ``cu_q``: the prompt form of
+    the MFMA kernel (bf16, Dk % 32 == 0, kv_rank % 16 == 0); without them that kernel takes one row per sequence
+    (decode steps).  Other shapes, fp32 and ``impl=1`` run the one-wave-per-(row, head) kernel.  Returns the
+    implementation used (0 MFMA, 1 wave)."""
     if _gpu(q):
         return _lat().latent_attn(q, cache, block_tables, row_seq, positions, float(scale), int(kv_rank), out, part_o,
-                                  part_ml)
-    return reference.latent_attn(q, cache, block_tables, row_seq, positions, scale, kv_rank, out)
+                                  part_ml, tiles, cu_q, LATENT_ATTN_IMPL if impl is None else int(impl))
+    reference.latent_attn(q, cache, block_tables, row_seq, positions, scale, kv_rank, out)
+    return 1
 
 
 def clamped_glu(gu, limit, alpha, out):

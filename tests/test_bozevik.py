@@ -56,6 +56,16 @@ def _cfg_b():
     ])
 
 
+def _cfg_c():
+    """Latent 48 + rotary 16 (a 64-wide cache row: the shapes the MFMA attention kernel takes in bf16), 5 and 18 heads."""
+    return O.make_config(width=64, vocab=128, eps=1e-5, logit_scale=0.8, layers=[
+        {"type": "latent_attention", "mixer": O.mixer(heads=5, dim=8, rot_dim=16, vdim=12, kv_rank=48, q_rank=24, base=1000.0, scale=0.3),
+         "mlp": O.dense(ff=64, limit=3.0)},
+        {"type": "latent_attention", "mixer": O.mixer(heads=18, dim=8, rot_dim=16, vdim=4, kv_rank=48, q_rank=40, base=1000.0, scale=0.25, kv_from=0),
+         "mlp": O.moe(experts=4, top=2, ff=32, limit=1.0, shared_ff=32, shared_limit=1.0)},
+    ])
+
+
 def _checkpoint(tmp_path, cfg, seed=0, tensors=None):
     from safetensors.torch import save_file
 
@@ -114,13 +124,13 @@ def _oracle(cfg, tensors, ids):
 # ---- whole prompts, decoding, portions ----------------------------------------------------------------
 @pytest.mark.parametrize("device", DEVICES)
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("make", [_cfg_a, _cfg_b])
+@pytest.mark.parametrize("make", [_cfg_a, _cfg_b, _cfg_c])
 def test_prompt_decode_and_portions_agree_with_oracle(tmp_path, device, dtype, make):
     device = _device(device)
     cfg = make()
     path, tensors = _checkpoint(tmp_path, cfg)
     eng = _engine(path, device, dtype)
-    ids = _tokens(3 * BS + 5, cfg["vocab"], 1)
+    ids = _tokens((3 if make is not _cfg_c else 9) * BS + 5, cfg["vocab"], 1)   # (_cfg_c: past one 64-row query tile)
     want = _oracle(cfg, tensors, ids)
     n = len(ids)
     plans = {
@@ -223,7 +233,7 @@ def test_latent_attn_op_picks_exactly_the_visible_keys(device, dtype):
     with scattered, non-monotonic block tables."""
     device = _device(device)
     g = torch.Generator().manual_seed(0)
-    H, r, rot, nb = 3, 24, 8, 12
+    H, r, rot, nb = 3, 48, 16, 12     # a 64-wide row: bf16 on the GPU takes the MFMA kernel, fp32 the wave kernel
     Dk = r + rot
     cache = (torch.randn(nb, BS, Dk, generator=g) * 0.1)
     table = torch.tensor([[7, 2, 9, 4, 11, 1], [3, 10, 5, 8, 6, 0]], dtype=torch.int32)
@@ -254,6 +264,56 @@ def test_latent_attn_op_picks_exactly_the_visible_keys(device, dtype):
             else:
                 base = torch.softmax(q[seq].to(dtype).float() @ cache.to(dtype).float()[table[seq].long()].reshape(-1, Dk)[: p + 1].t(), -1)
                 assert torch.allclose(w, base)                # ... and one past the query changes nothing
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("H,r,rot", [(1, 16, 16), (5, 48, 16), (20, 128, 32), (70, 64, 64)])
+def test_latent_attn_mfma_forms_against_the_wave_kernel(H, r, rot):
+    """Prompt tiles (several runs that start mid-sequence, partial 64-row tiles, scattered blocks) and the decode form
+    with split-KV partitions, MFMA kernel vs the one-wave kernel and vs a plain softmax."""
+    if not torch.cuda.is_available():
+        pytest.skip("no GPU")
+    dev, g = "cuda", torch.Generator().manual_seed(H)
+    Dk, bs, nb = r + rot, 16, 80
+    cache = torch.randn(nb, bs, Dk, generator=g).to(torch.bfloat16)
+    runs = [(300, 130), (0, 70), (517, 1), (64, 64)]                      # (first position, rows) per sequence
+    perm = torch.randperm(nb - 1, generator=g) + 1
+    mb = 40
+    table = torch.zeros(len(runs), mb, dtype=torch.int32)
+    used = 0
+    for i, (p0, n) in enumerate(runs):
+        need = -(-(p0 + n) // bs)
+        table[i, :need] = perm[used % 8:used % 8 + need].int()          # overlapping block sets are fine for a read-only op
+        used += 3
+    pos = torch.cat([torch.arange(p0, p0 + n) for p0, n in runs]).int()
+    row_seq = torch.cat([torch.full((n,), i) for i, (_, n) in enumerate(runs)]).int()
+    cu = torch.tensor([0] + list(torch.tensor([n for _, n in runs]).cumsum(0)), dtype=torch.int32)
+    tiles = torch.tensor([(i, o) for i, (_, n) in enumerate(runs) for o in range(0, n, 64)] + [(0, 1 << 24)], dtype=torch.int32)
+    T = int(pos.numel())
+    q = (torch.randn(T, H, Dk, generator=g) * 0.5).to(torch.bfloat16)
+    scale = 0.2
+    want = torch.zeros(T, H, r)
+    flat = cache.float()
+    for t in range(T):
+        rows = flat[table[row_seq[t]].long()].reshape(-1, Dk)[: int(pos[t]) + 1]
+        want[t] = torch.softmax(q[t].float() @ rows.t() * scale, -1) @ rows[:, :r]
+    d = lambda t: t.to(dev)
+    outs = {}
+    for name, kw in {"wave": dict(impl=1), "tiles": dict(tiles=d(tiles), cu_q=d(cu), impl=0), "rows": dict(impl=0)}.items():
+        o = torch.zeros(T, H, r, dtype=torch.bfloat16, device=dev)
+        used_impl = ops.latent_attn(d(q), d(cache), d(table), d(row_seq), d(pos), scale, r, o, **kw)
+        assert used_impl == (1 if name == "wave" else 0)
+        outs[name] = o.float().cpu()
+        assert float((outs[name] - want).abs().max()) < 3e-2, name
+    # split-KV partitions (decode form): rows of different sequences, context far past one partition
+    parts = -(-(mb * bs) // ops.LATENT_ATTN_PART)
+    sel = torch.tensor([129, 130 + 69, 200, 201 + 63])                    # last rows of the four runs
+    for impl in (0, 1):
+        o = torch.zeros(4, H, r, dtype=torch.bfloat16, device=dev)
+        po = torch.zeros(4, H, parts, r, device=dev)
+        pml = torch.zeros(4, H, parts, 2, device=dev)
+        ops.latent_attn(d(q[sel]), d(cache), d(table), d(torch.arange(4).int()), d(pos[sel]), scale, r, o, po, pml, impl=impl)
+        assert float((o.float().cpu() - want[sel]).abs().max()) < 3e-2, impl
 
 
 # ---- each mechanism alone: op vs oracle function ------------------------------------------------------
