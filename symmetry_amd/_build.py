@@ -95,9 +95,9 @@ HIP_FLAGS = [
     "-ffp-contract=fast",
     "-munsafe-fp-atomics",
     "-Wno-unused-result",
-    # no packed-fp32 instruction selection (v_pk_*_f32): scalar fp32 code only
-    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
 ]
+# no packed-fp32 instruction selection (v_pk_*_f32): scalar fp32 code only
+NO_PACKED_FP32 = ["-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
 
 
 def build_kernels(verbose: bool = False, force: bool = False) -> str:
@@ -150,7 +150,7 @@ def build_latent(verbose: bool = False, force: bool = False) -> str:
         src, obj = os.path.join(kdir, name), os.path.join(OBJ, name + ".o")
         objs.append(obj)
         if force or _newer(obj, [src] + headers):
-            jobs.append([HIPCC, "-c", src, "-o", obj, "-I", kdir] + HIP_FLAGS)
+            jobs.append([HIPCC, "-c", src, "-o", obj, "-I", kdir] + HIP_FLAGS + NO_PACKED_FP32)
     for name in LATENT_BINDINGS:
         src, obj = os.path.join(CSRC, "bindings", name), os.path.join(OBJ, "bind_" + name + ".o")
         objs.append(obj)
