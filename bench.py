@@ -70,6 +70,10 @@ def _args():
     ap.add_argument("--client-end", type=int, default=1, help="1: also measure at the client sockets")
     ap.add_argument("--client-tokens", type=int, default=256, help="tokens per client in the client-end run")
     ap.add_argument("--no-graphs", action="store_true")
+    ap.add_argument("--families", action="store_true",
+                    help="instead of the serving benchmark: prefill / decode throughput of Bozevik stacks beside the "
+                         "closest Llama / Mixtral stacks of equal size (bench/families.py; one GPU)")
+    ap.add_argument("--family-sizes", default="w2048,w4096,moe-w2048")
     ap.add_argument("--nt-weights", type=int, default=None, help="A/B: non-temporal decode weight loads (0/1)")
     ap.add_argument("--max-batched-tokens", type=int, default=None, help="A/B: token budget of a pure-prefill step")
     ap.add_argument("--mixed-prefill-tokens", type=int, default=None, help="A/B: prompt budget of mixed steps")
@@ -175,6 +179,11 @@ def _self_launch(args) -> int | None:
 
 def main() -> int:
     args = _args()
+    if args.families:
+        sys.path.insert(0, os.path.join(os.path.dirname(os.path.abspath(__file__)), "bench"))
+        import families
+
+        return families.main(["--sizes", args.family_sizes])
     code = _self_launch(args)
     if code is not None:
         return code

@@ -206,14 +206,18 @@ int64_t latent_attn(const Tensor& q, const Tensor& cache, const Tensor& block_ta
                   out.numel() == (int64_t)a.T * a.H * kv_rank && row_seq.numel() >= a.T && positions.numel() >= a.T &&
                   a.H <= 65535, "latent_attn: shapes");
   a.parts = 1;
+  a.part_tokens = 32;
   if (part_o.has_value()) {
+    // partials [T, H, parts, kv_rank] + [T, H, parts, 2]: the caller's `parts` partitions cover the block-table span
     TORCH_CHECK(part_ml.has_value(), "latent_attn: part_o without part_ml");
     dtype(*part_o, at::kFloat, "part_o");
     dtype(*part_ml, at::kFloat, "part_ml");
+    TORCH_CHECK(part_o->dim() == 4 && part_o->size(0) == a.T && part_o->size(1) == a.H && part_o->size(3) == kv_rank &&
+                    part_ml->numel() == (int64_t)a.T * a.H * part_o->size(2) * 2, "latent_attn: partial buffer shapes");
+    a.parts = (int)part_o->size(2);
     const int64_t span = (int64_t)a.max_blocks * a.BS;
-    a.parts = (int)((span + latent_attn_part_tokens() - 1) / latent_attn_part_tokens());
-    TORCH_CHECK(part_o->numel() >= (int64_t)a.T * a.H * a.parts * kv_rank && part_ml->numel() >= (int64_t)a.T * a.H * a.parts * 2 &&
-                    a.parts <= 65535, "latent_attn: partial buffers too small");
+    a.part_tokens = (int)(((span + a.parts - 1) / a.parts + 31) / 32 * 32);
+    TORCH_CHECK(a.parts >= 1 && a.parts <= 1024 && (int64_t)a.parts * a.part_tokens >= span, "latent_attn: partitions");
     a.part_o = ptr<float>(*part_o);
     a.part_ml = ptr<float>(*part_ml);
   }
@@ -239,8 +243,6 @@ int64_t latent_attn(const Tensor& q, const Tensor& cache, const Tensor& block_ta
                   (reinterpret_cast<uintptr_t>(out.data_ptr()) % 16 == 0), "latent_attn: 16-byte aligned tensors");
   return launch_latent_attn(a, f32, (int)impl, cur_stream(q));
 }
-
-int64_t latent_attn_part() { return latent_attn_part_tokens(); }
 
 void clamped_glu(const Tensor& gu, double limit, double alpha, Tensor& out) {
   const int f32 = act(gu, "gu");
@@ -334,7 +336,6 @@ TORCH_LIBRARY(symmetry_amd_latent, m) {
       "latent_attn(Tensor q, Tensor cache, Tensor block_tables, Tensor row_seq, Tensor positions, float scale, "
       "int kv_rank, Tensor(a!) out, Tensor(b!)? part_o, Tensor(c!)? part_ml, Tensor? tiles, Tensor? cu_q, int impl) -> int",
       &latent_attn);
-  m.def("latent_attn_part() -> int", &latent_attn_part);
   m.def("clamped_glu(Tensor gu, float limit, float alpha, Tensor(a!) out) -> ()", &clamped_glu);
   m.def("sigmoid_topk(Tensor x, Tensor Wr, int k, Tensor(a!) ids, Tensor(b!) w) -> ()", &sigmoid_topk);
   m.def("expert_offsets(Tensor ids, int R, int E, Tensor(a!) offsets, Tensor(b!) cursor) -> ()", &expert_offsets);

@@ -118,7 +118,6 @@ SYM_DEV float dot_row(const float* q, const float* r, int n) {
   return s;
 }
 
-constexpr int PART = 256;  // keys per split-KV partition of the decode form
 
 // One wave per (query row, head, key partition).  Each lane scores one key of a 64-key tile (the query in LDS, the
 // cache row streamed), the tile's softmax statistics are wave reductions, and the weighted sum of the latents
@@ -131,8 +130,8 @@ __global__ __launch_bounds__(64) void latent_attn_wave_kernel(LatentAttnArgs a) 
   const int row = blockIdx.x, h = blockIdx.y, part = blockIdx.z;
   const int lane = threadIdx.x;
   const int nkeys = a.positions[row] + 1;
-  const int k0 = a.parts > 1 ? part * PART : 0;
-  const int k1 = a.parts > 1 ? min(nkeys, k0 + PART) : nkeys;
+  const int k0 = a.parts > 1 ? part * a.part_tokens : 0;
+  const int k1 = a.parts > 1 ? min(nkeys, k0 + a.part_tokens) : nkeys;
   const T* q = (const T*)a.q + ((long long)row * a.H + h) * a.Dk;
   for (int c = lane; c < a.Dk; c += 64) qs[c] = (float)q[c];
   __syncthreads();
@@ -192,51 +191,73 @@ __global__ __launch_bounds__(64) void latent_attn_wave_kernel(LatentAttnArgs a) 
   }
 }
 
+// Combine the split-KV partials of one (row, head): one wave; the per-partition weights exp(m_p - m) / l are
+// computed once (lanes over partitions, kept in LDS), then the lanes stride over the latent dims.
 template <typename T>
 __global__ __launch_bounds__(64) void latent_attn_merge_kernel(LatentAttnArgs a) {
+  __shared__ float wp[1024];
   const int row = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
   const long long p0 = ((long long)row * a.H + h) * a.parts;
-  const int np = min(a.parts, (a.positions[row] + PART) / PART);  // partitions that hold keys of this row
+  const int np = min(a.parts, (a.positions[row] + a.part_tokens) / a.part_tokens);  // partitions that hold keys
   float m = -INFINITY;
-  for (int p = 0; p < np; ++p) m = fmaxf(m, a.part_ml[2 * (p0 + p)]);
+  for (int p = lane; p < np; p += 64) m = fmaxf(m, a.part_ml[2 * (p0 + p)]);
+  m = wave_max(m);
   float l = 0.f;
-  for (int p = 0; p < np; ++p) l += a.part_ml[2 * (p0 + p) + 1] * expf(a.part_ml[2 * (p0 + p)] - m);
+  for (int p = lane; p < np; p += 64) {
+    const float w = __expf(a.part_ml[2 * (p0 + p)] - m);
+    wp[p] = w;
+    l += a.part_ml[2 * (p0 + p) + 1] * w;
+  }
+  l = wave_sum(l);
+  __syncthreads();
+  const float inv = 1.f / l;
   T* out = (T*)a.out + ((long long)row * a.H + h) * a.kv_rank;
   for (int c = lane; c < a.kv_rank; c += 64) {
     float acc = 0.f;
-    for (int p = 0; p < np; ++p) acc += a.part_o[(p0 + p) * a.kv_rank + c] * expf(a.part_ml[2 * (p0 + p)] - m);
-    out[c] = (T)(acc / l);
+    for (int p = 0; p < np; ++p) acc += a.part_o[(p0 + p) * a.kv_rank + c] * wp[p];
+    out[c] = (T)(acc * inv);
   }
 }
-
 
 constexpr int KT = 32;        // keys per staged tile
 constexpr int LDV = KT + 4;   // row pitch (elements) of the transposed latent tile
 
-template <int NKM, int RTM, bool DECODE>
-__global__ __launch_bounds__(256) void latent_attn_mfma_kernel(LatentAttnArgs a) {
+// NW waves per workgroup, 16 query vectors each.  Prompt form (DECODE = false): NW = 4, a tile of 64 rows of one head.
+// Decode form: one row, 16 * NW of its heads (NW = 1, 2, 4 by the head count), one key partition per workgroup.
+// The next tile's cache rows are fetched into registers while the current tile is multiplied (the global latency
+// hides behind the MFMAs); they go to LDS between two barriers at the top of the next iteration.
+template <int NKM, int RTM, bool DECODE, int NW>
+__global__ __launch_bounds__(64 * NW) void latent_attn_mfma_kernel(LatentAttnArgs a) {
   extern __shared__ __attribute__((aligned(16))) char smem[];
+  constexpr int NTH = 64 * NW;
+  constexpr int CSTEP = NTH / 32;                       // 16-byte chunks of a row taken per pass of the workgroup
+  constexpr int CHM = (NKM * 4 + CSTEP - 1) / CSTEP;    // passes (chunks per thread)
+  // up to 9 passes stay in registers across the multiply (prefetch); workgroups of fewer waves have more passes per
+  // thread than registers to spare and stage in batches instead (no prefetch: they run one or two tiles)
+  constexpr bool PREFETCH = CHM <= 9;
+  constexpr int NB = PREFETCH ? CHM : 9;
   const int Dk = a.Dk, r = a.kv_rank, H = a.H;
-  const int nk = Dk >> 5, rt = r >> 4;
+  const int nk = Dk >> 5, rt = r >> 4, nchunk = Dk >> 3;
   const int ldk = Dk + 8;
   bf16* Ks = reinterpret_cast<bf16*>(smem);  // [KT][ldk] key-major cache rows
   bf16* Vt = Ks + KT * ldk;                   // [r][LDV] latent part, dim-major
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int n = lane & 15, g = lane >> 4;
-  int seq, qrow, head, limit, k_lo, k_hi, wave_hi, part = 0;
+  int seq, qrow, head, limit, k_lo, k_hi, wave_hi, wave_lo, part = 0;  // wave_lo: keys every query vector of the wave sees
   bool valid, wave_active;
   if constexpr (DECODE) {
     qrow = blockIdx.x;
     seq = a.row_seq[qrow];
-    head = blockIdx.y * 64 + wave * 16 + n;
+    head = blockIdx.y * 16 * NW + wave * 16 + n;
     valid = head < H;
-    wave_active = blockIdx.y * 64 + wave * 16 < H;
+    wave_active = blockIdx.y * 16 * NW + wave * 16 < H;
     limit = a.positions[qrow];
     part = blockIdx.z;
-    k_lo = a.parts > 1 ? part * PART : 0;
-    k_hi = a.parts > 1 ? min(limit + 1, k_lo + PART) : limit + 1;
+    k_lo = a.parts > 1 ? part * a.part_tokens : 0;
+    k_hi = a.parts > 1 ? min(limit + 1, k_lo + a.part_tokens) : limit + 1;
     if (k_lo >= k_hi) return;  // a partition past this row's keys: the merge never reads it
     wave_hi = k_hi;
+    wave_lo = limit + 1;
   } else {
     seq = a.tiles[2 * blockIdx.x];
     const int off = a.tiles[2 * blockIdx.x + 1];
@@ -249,8 +270,9 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_kernel(LatentAttnArgs a)
     head = blockIdx.y;
     limit = a.positions[qrow];
     k_lo = 0;
-    k_hi = a.positions[q0 + min(off + 63, qlen - 1)] + 1;       // a run's rows are consecutive positions
+    k_hi = a.positions[q0 + min(off + 16 * NW - 1, qlen - 1)] + 1;       // a run's rows are consecutive positions
     wave_hi = a.positions[q0 + min(off + wave * 16 + 15, qlen - 1)] + 1;
+    wave_lo = a.positions[q0 + min(off + wave * 16, qlen - 1)] + 1;
   }
   const bf16* qp = (const bf16*)a.q + ((long long)qrow * H + min(head, H - 1)) * Dk;
   bf16x8 qf[NKM];
@@ -263,15 +285,24 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_kernel(LatentAttnArgs a)
   float m = -INFINITY, l = 0.f;
   const int* bt = a.block_tables + (long long)seq * a.max_blocks;
   const bf16* cache = (const bf16*)a.cache;
-  const int key_in = tid & 31;
-  for (int k0 = k_lo; k0 < k_hi; k0 += KT) {
-    __syncthreads();  // the previous tile's fragment reads are done
-    {
-      const int key = min(k0 + key_in, k_hi - 1);
-      const bf16* src = cache + ((long long)bt[key / a.BS] * a.BS + key % a.BS) * Dk;
-      for (int c = tid >> 5; c < (Dk >> 3); c += 8) {
+  const int key_in = tid & 31, c0 = tid >> 5;
+  uint4 pre[NB];
+  auto fetch = [&](int k0, int i0) {
+    const int key = min(k0 + key_in, k_hi - 1);
+    const bf16* src = cache + ((long long)bt[key / a.BS] * a.BS + key % a.BS) * Dk;
+#pragma unroll
+    for (int i = 0; i < NB; ++i) {
+      const int c = c0 + (i0 + i) * CSTEP;
+      if (c < nchunk) pre[i] = *reinterpret_cast<const uint4*>(src + c * 8);
+    }
+  };
+  auto stash = [&](int i0) {
+#pragma unroll
+    for (int i = 0; i < NB; ++i) {
+      const int c = c0 + (i0 + i) * CSTEP;
+      if (c < nchunk) {
         Pack8 pk;
-        pk.u = *reinterpret_cast<const uint4*>(src + c * 8);
+        pk.u = pre[i];
         *reinterpret_cast<uint4*>(Ks + key_in * ldk + c * 8) = pk.u;
         if (c * 8 < r) {
 #pragma unroll
@@ -279,47 +310,81 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_kernel(LatentAttnArgs a)
         }
       }
     }
+  };
+  if constexpr (PREFETCH) fetch(k_lo, 0);
+  for (int k0 = k_lo; k0 < k_hi; k0 += KT) {
+    __syncthreads();  // the previous tile's fragment reads are done
+    if constexpr (PREFETCH) {
+      stash(0);
+    } else {
+      for (int i0 = 0; i0 < CHM; i0 += NB) {
+        fetch(k0, i0);
+        stash(i0);
+      }
+    }
     __syncthreads();
+    if constexpr (PREFETCH)
+      if (k0 + KT < k_hi) fetch(k0 + KT, 0);
     if (!wave_active || k0 >= wave_hi) continue;
     // S^T: rows = keys (sub * 16 + g * 4 + i), column = this lane's query vector n
+    // (four independent accumulator chains: both 16-key subtiles, even and odd k steps)
     f32x4 st[2];
+    {
+      f32x4 acc[4];
 #pragma unroll
-    for (int sub = 0; sub < 2; ++sub) {
-      f32x4 acc = {0.f, 0.f, 0.f, 0.f};
-      const bf16* kr = Ks + (sub * 16 + n) * ldk + g * 8;
+      for (int i = 0; i < 4; ++i) acc[i] = f32x4{0.f, 0.f, 0.f, 0.f};
+      const bf16* kr = Ks + n * ldk + g * 8;
 #pragma unroll
       for (int s = 0; s < NKM; ++s)
-        if (s < nk) acc = mfma16(*reinterpret_cast<const bf16x8*>(kr + s * 32), qf[s], acc);
-      st[sub] = acc;
+        if (s < nk) {
+          acc[s & 1] = mfma16(*reinterpret_cast<const bf16x8*>(kr + s * 32), qf[s], acc[s & 1]);
+          acc[2 + (s & 1)] = mfma16(*reinterpret_cast<const bf16x8*>(kr + 16 * ldk + s * 32), qf[s], acc[2 + (s & 1)]);
+        }
+      st[0] = acc[0] + acc[1];
+      st[1] = acc[2] + acc[3];
     }
+    // scale; mask only where a tile reaches past some query vector's last key (the diagonal tiles, the range's tail)
+    const bool edge = k0 + KT > wave_lo || k0 + KT > k_hi;  // wave-uniform
     float mx = -INFINITY;
 #pragma unroll
     for (int sub = 0; sub < 2; ++sub)
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        const int key = k0 + sub * 16 + g * 4 + i;
-        const float v = (key > limit || key >= k_hi) ? -INFINITY : st[sub][i] * a.scale;
+        float v = st[sub][i] * a.scale;
+        if (edge) {
+          const int key = k0 + sub * 16 + g * 4 + i;
+          if (key > limit || key >= k_hi) v = -INFINITY;
+        }
         st[sub][i] = v;
         mx = fmaxf(mx, v);
       }
     mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
     mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-    const float m_new = fmaxf(m, mx);          // finite: every query vector sees the first key of its range
-    const float alpha = __expf(m - m_new);
+    // deferred rescale: the running maximum moves (and the accumulators are rescaled, a pass over every accumulator
+    // register) only when some query vector's maximum grew by more than 8; until then weights may reach e^8, which
+    // fp32 sums and bf16 products hold as well as values below 1.  The first tile always takes the branch.
+    if (__any(mx > m + 8.f)) {
+      const float m_new = fmaxf(m, mx);        // finite: every query vector sees the first key of its range
+      const float alpha = __expf(m - m_new);
+      l *= alpha;
+#pragma unroll
+      for (int dt = 0; dt < RTM; ++dt)
+        if (dt < rt) o[dt] = o[dt] * alpha;
+      m = m_new;
+    }
     float ps = 0.f;
     Pack8 pb;
 #pragma unroll
     for (int sub = 0; sub < 2; ++sub)
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        const float p = __expf(st[sub][i] - m_new);
+        const float p = __expf(st[sub][i] - m);
         ps += p;
         pb.h[sub * 4 + i] = (bf16)p;
       }
     ps += __shfl_xor(ps, 16, 64);
     ps += __shfl_xor(ps, 32, 64);
-    l = l * alpha + ps;
-    m = m_new;
+    l += ps;
     // O^T += V^T P^T: k index g * 8 + j of the product is key g * 4 + j (j < 4) / 16 + g * 4 + j - 4 of the tile
     const bf16* vr = Vt + n * LDV + g * 4;
 #pragma unroll
@@ -329,7 +394,7 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_kernel(LatentAttnArgs a)
         const uint2 lo = *reinterpret_cast<const uint2*>(vr + dt * 16 * LDV);
         const uint2 hi = *reinterpret_cast<const uint2*>(vr + dt * 16 * LDV + 16);
         va.u = make_uint4(lo.x, lo.y, hi.x, hi.y);
-        o[dt] = mfma16(va.v, pb.v, o[dt] * alpha);
+        o[dt] = mfma16(va.v, pb.v, o[dt]);
       }
   }
   if (!valid) return;
@@ -358,26 +423,34 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_kernel(LatentAttnArgs a)
   }
 }
 
-template <int NKM, int RTM>
-void mfma_launch(const LatentAttnArgs& a, hipStream_t s) {
+template <int NKM, int RTM, bool DECODE, int NW>
+void mfma_launch_one(const LatentAttnArgs& a, dim3 grid, hipStream_t s) {
   const size_t lds = ((size_t)KT * (a.Dk + 8) + (size_t)a.kv_rank * LDV) * sizeof(bf16);
   static bool raised = false;  // (per instantiation) dynamic LDS beyond the 64 KB default
   if (!raised) {
-    hipFuncSetAttribute(reinterpret_cast<const void*>(&latent_attn_mfma_kernel<NKM, RTM, true>),
-                        hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024);
-    hipFuncSetAttribute(reinterpret_cast<const void*>(&latent_attn_mfma_kernel<NKM, RTM, false>),
+    hipFuncSetAttribute(reinterpret_cast<const void*>(&latent_attn_mfma_kernel<NKM, RTM, DECODE, NW>),
                         hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024);
     raised = true;
   }
-  if (a.tiles)
-    latent_attn_mfma_kernel<NKM, RTM, false><<<dim3(a.ntiles, a.H), 256, lds, s>>>(a);
-  else
-    latent_attn_mfma_kernel<NKM, RTM, true><<<dim3(a.T, (a.H + 63) / 64, a.parts), 256, lds, s>>>(a);
+  latent_attn_mfma_kernel<NKM, RTM, DECODE, NW><<<grid, 64 * NW, lds, s>>>(a);
+}
+
+template <int NKM, int RTM>
+void mfma_launch(const LatentAttnArgs& a, hipStream_t s) {
+  if (a.tiles) {
+    mfma_launch_one<NKM, RTM, false, 4>(a, dim3(a.ntiles, a.H), s);
+  } else if (a.H <= 16) {
+    mfma_launch_one<NKM, RTM, true, 1>(a, dim3(a.T, (a.H + 15) / 16, a.parts), s);
+  } else if (a.H <= 32) {
+    mfma_launch_one<NKM, RTM, true, 2>(a, dim3(a.T, (a.H + 31) / 32, a.parts), s);
+  } else {
+    mfma_launch_one<NKM, RTM, true, 4>(a, dim3(a.T, (a.H + 63) / 64, a.parts), s);
+  }
 }
 
 bool mfma_dispatch(const LatentAttnArgs& a, hipStream_t s) {
   const int nk = a.Dk / 32, rt = a.kv_rank / 16;
-  if (a.Dk % 32 || a.kv_rank % 16 || nk > 18 || rt > 32) return false;
+  if (a.Dk % 32 || a.kv_rank % 16 || nk > 18 || rt > 32 || a.part_tokens % KT) return false;
   if (nk <= 5 && rt <= 8) mfma_launch<5, 8>(a, s);
   else if (nk <= 10 && rt <= 16) mfma_launch<10, 16>(a, s);
   else mfma_launch<18, 32>(a, s);
@@ -397,7 +470,6 @@ void attn_dispatch(const LatentAttnArgs& a, hipStream_t s) {
 
 }  // namespace
 
-int latent_attn_part_tokens() { return PART; }
 
 void launch_latent_prep(const LatentPrepArgs& a, int T, int f32, hipStream_t s) {
   if (T <= 0) return;

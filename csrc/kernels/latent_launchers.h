@@ -51,7 +51,8 @@ struct LatentAttnArgs {
   void* out;            // [T][H][kv_rank]: softmax-weighted sum of the latents
   float* part_o;        // split-KV partials (decode form): [T][H][parts][kv_rank], [T][H][parts][2]
   float* part_ml;
-  int T, H, Dk, kv_rank, BS, max_blocks, parts;
+  int T, H, Dk, kv_rank, BS, max_blocks;
+  int parts, part_tokens;  // split-KV: partition p of a row covers keys [p * part_tokens, (p + 1) * part_tokens)
   float scale;
   // prompt form of the MFMA kernel: 64-row query tiles (sequence, first row within the sequence's run) over the
   // runs cu_q[seq] .. cu_q[seq + 1]; nullptr: one query row per sequence (decode steps)
@@ -62,7 +63,6 @@ struct LatentAttnArgs {
 // impl: 0 = MFMA kernel where the shapes allow (bf16, Dk % 32 == 0, kv_rank % 16 == 0, Dk <= 576, kv_rank <= 512),
 // 1 = always the one-wave-per-(row, head) kernel (all shapes, both dtypes).  Returns the implementation used.
 int launch_latent_attn(const LatentAttnArgs& a, int f32, int impl, hipStream_t s);
-int latent_attn_part_tokens();
 
 // ---- glu_moe.hip -------------------------------------------------------------------------------------
 // gu [R][2F] = gate | up  ->  out [R][F] = g' * sigmoid(alpha * g') * (u' + 1), g' = min(g, limit), u' = clamp(u, +-limit)

@@ -48,7 +48,9 @@ __global__ __launch_bounds__(NT) void token_shift_kernel(const float* __restrict
   }
 }
 
-template <typename T, typename TD>
+// EPT > 0: the row's delta, x and weight are read once into registers (d <= NT * EPT), all loads in flight together;
+// EPT == 0: any width, the delta row is re-read for each pass (it stays in L1 / L2).
+template <typename T, typename TD, int EPT>
 __global__ __launch_bounds__(NT) void add_layer_norm_kernel(const TD* __restrict__ delta, const T* __restrict__ w,
                                                             float eps, float* __restrict__ x,
                                                             const int* __restrict__ save, float* __restrict__ state,
@@ -58,21 +60,43 @@ __global__ __launch_bounds__(NT) void add_layer_norm_kernel(const TD* __restrict
   __shared__ float scratch[NT / 64];
   const int row = blockIdx.x;
   const TD* dr = delta + (long long)row * d;
+  float* xr = x + (long long)row * d;
+  constexpr int NR = EPT > 0 ? EPT : 1;
+  float dv[NR], xv[NR], wv[NR];
   float sum = 0.f;
-  for (int c = threadIdx.x; c < d; c += NT) sum += (float)dr[c];
+  if constexpr (EPT > 0) {
+#pragma unroll
+    for (int i = 0; i < EPT; ++i) {
+      const int c = threadIdx.x + i * NT;
+      const bool in = c < d;
+      dv[i] = in ? (float)dr[c] : 0.f;
+      xv[i] = in ? xr[c] : 0.f;
+      wv[i] = in ? (float)w[c] : 0.f;
+      sum += dv[i];
+    }
+  } else {
+    for (int c = threadIdx.x; c < d; c += NT) sum += (float)dr[c];
+  }
   const float mean = block_sum<NT>(sum, scratch) / (float)d;
   float sq = 0.f;
-  for (int c = threadIdx.x; c < d; c += NT) {
-    const float v = (float)dr[c] - mean;
-    sq += v * v;
+  if constexpr (EPT > 0) {
+#pragma unroll
+    for (int i = 0; i < EPT; ++i) {
+      const float v = threadIdx.x + i * NT < d ? dv[i] - mean : 0.f;
+      sq += v * v;
+    }
+  } else {
+    for (int c = threadIdx.x; c < d; c += NT) {
+      const float v = (float)dr[c] - mean;
+      sq += v * v;
+    }
   }
   const float rstd = 1.f / sqrtf(block_sum<NT>(sq, scratch) / (float)d + eps);
   const int sv = save ? save[row] : -1;
-  for (int c = threadIdx.x; c < d; c += NT) {
+  auto finish = [&](int c, float dl, float xo, float wc) {
     const long long o = (long long)row * d + c;
-    const float xo = x[o];
     if (sv >= 0) state[(long long)sv * state_stride + c] = xo;
-    float xn = xo + ((float)dr[c] - mean) * rstd * (float)w[c];
+    float xn = xo + (dl - mean) * rstd * wc;
     if (hist) {
       hist[(long long)hist_idx * hist_stride + o] = xn;
       float m = coef[hist_idx] * xn;
@@ -81,6 +105,15 @@ __global__ __launch_bounds__(NT) void add_layer_norm_kernel(const TD* __restrict
     }
     x[o] = xn;
     if (out_act) out_act[o] = (T)xn;
+  };
+  if constexpr (EPT > 0) {
+#pragma unroll
+    for (int i = 0; i < EPT; ++i) {
+      const int c = threadIdx.x + i * NT;
+      if (c < d) finish(c, dv[i], xv[i], wv[i]);
+    }
+  } else {
+    for (int c = threadIdx.x; c < d; c += NT) finish(c, (float)dr[c], xr[c], (float)w[c]);
   }
 }
 
@@ -122,22 +155,34 @@ void launch_token_shift(const float* x, const void* mu, const int* prev_row, con
     token_shift_kernel<bf16><<<T, NT, 0, s>>>(x, (const bf16*)mu, prev_row, state, state_stride, (bf16*)h, d);
 }
 
+template <typename T, typename TD>
+void add_layer_norm_pick(const void* delta, const void* w, float eps, float* x, const int* save, float* state,
+                         long long state_stride, float* hist, long long hist_stride, const float* coef, int hist_idx,
+                         void* out_act, int T_, int d, hipStream_t s) {
+#define SYM_ALN(EPT)                                                                                                   \
+  add_layer_norm_kernel<T, TD, EPT><<<T_, NT, 0, s>>>((const TD*)delta, (const T*)w, eps, x, save, state, state_stride, \
+                                                      hist, hist_stride, coef, hist_idx, (T*)out_act, d)
+  if (d <= NT * 4) SYM_ALN(4);
+  else if (d <= NT * 8) SYM_ALN(8);
+  else if (d <= NT * 16) SYM_ALN(16);
+  else if (d <= NT * 32) SYM_ALN(32);
+  else SYM_ALN(0);
+#undef SYM_ALN
+}
+
 void launch_add_layer_norm(const void* delta, int delta_f32, const void* w, float eps, float* x, const int* save,
                            float* state, long long state_stride, float* hist, long long hist_stride, const float* coef,
                            int hist_idx, void* out_act, int T, int d, int f32, hipStream_t s) {
   if (T <= 0) return;
   if (f32)
-    add_layer_norm_kernel<float, float><<<T, NT, 0, s>>>((const float*)delta, (const float*)w, eps, x, save, state,
-                                                        state_stride, hist, hist_stride, coef, hist_idx,
-                                                        (float*)out_act, d);
+    add_layer_norm_pick<float, float>(delta, w, eps, x, save, state, state_stride, hist, hist_stride, coef, hist_idx,
+                                      out_act, T, d, s);
   else if (delta_f32)
-    add_layer_norm_kernel<bf16, float><<<T, NT, 0, s>>>((const float*)delta, (const bf16*)w, eps, x, save, state,
-                                                       state_stride, hist, hist_stride, coef, hist_idx,
-                                                       (bf16*)out_act, d);
+    add_layer_norm_pick<bf16, float>(delta, w, eps, x, save, state, state_stride, hist, hist_stride, coef, hist_idx,
+                                     out_act, T, d, s);
   else
-    add_layer_norm_kernel<bf16, bf16><<<T, NT, 0, s>>>((const bf16*)delta, (const bf16*)w, eps, x, save, state,
-                                                      state_stride, hist, hist_stride, coef, hist_idx, (bf16*)out_act,
-                                                      d);
+    add_layer_norm_pick<bf16, bf16>(delta, w, eps, x, save, state, state_stride, hist, hist_stride, coef, hist_idx,
+                                    out_act, T, d, s);
 }
 
 void launch_layer_norm(const float* x, const long long* rows, const void* w, float eps, void* out, int n, int d,

@@ -162,6 +162,16 @@ class BozevikLM:
         ops.clamped_glu(gu, spec.limit, GLU_ALPHA, act)
         return self._linear(name + ".down", act, f["w_down"])
 
+    def _grouped(self, xs: torch.Tensor, W: torch.Tensor, offsets: torch.Tensor, y: torch.Tensor) -> None:
+        """y = xs @ W[e]^T over the expert segments: the main kernel library's MFMA grouped GEMM (bf16, shapes that
+        tile for it: K % 64, N % 128, at most 64 experts) where that library is built, else the all-shapes kernel."""
+        E, N, K = W.shape
+        if (self.dtype == torch.bfloat16 and self.device.type != "cpu" and not ops.torch_mode() and E <= 64
+                and K % 64 == 0 and N % 128 == 0 and ops.native_available()):
+            ops.grouped_gemm(xs, W, offsets, 0, y, ops.GROUPED_BF16)
+        else:
+            ops.grouped_linear(xs, W, offsets, y)
+
     def _moe(self, P: dict, x: torch.Tensor) -> torch.Tensor:
         """Routed feed-forward: fp32 sigmoid scores, top-k, each chosen expert applied to (score * x), plus the shared
         expert; returns the fp32 sum.  Segment bounds stay on the device (no host sync: graph-capturable)."""
@@ -179,11 +189,11 @@ class BozevikLM:
         ops.scatter_scaled(x, ids, wts, k, offsets, cursor, xs, dst)
         F = spec.expert.ff
         y1 = self._buf("moe.y1", (R, 2 * F))
-        ops.grouped_linear(xs, P["w13"], offsets, y1)
+        self._grouped(xs, P["w13"], offsets, y1)
         act = self._buf("moe.act", (R, F))
         ops.clamped_glu(y1, spec.expert.limit, GLU_ALPHA, act)
         y2 = self._buf("moe.y2", (R, d))
-        ops.grouped_linear(act, P["w2"], offsets, y2)
+        self._grouped(act, P["w2"], offsets, y2)
         shared = self._glu("moe.shared", x, P["shared"], spec.shared) if P["shared"] is not None else None
         out = self._buf("moe.out", (T, d), torch.float32)
         ops.gather_sum(y2, dst, k, shared, out)
@@ -205,7 +215,7 @@ class BozevikLM:
         olat = self._buf("olat", (T, H, r))
         part_o = part_ml = None
         if b.kind == "decode" and self.device.type != "cpu":
-            parts = -(-(b.block_tables.shape[1] * cache.block_size) // ops.LATENT_ATTN_PART)
+            parts = ops.latent_attn_parts(T, b.block_tables.shape[1] * cache.block_size)
             if parts > 1:
                 part_o = self._buf("attn.part_o", (T, H, parts, r), torch.float32)
                 part_ml = self._buf("attn.part_ml", (T, H, parts, 2), torch.float32)

@@ -225,9 +225,9 @@ def bozevik_to_config(c: BozevikConfig) -> dict:
 
 
 def _bozevik_stack(name, vocab, width, n_layers, heads, dim, rot_dim, vdim, kv_rank, q_rank, ff, experts=0, top=2,
-                   expert_ff=0, shared_ff=0, share_every=2, **kw) -> BozevikConfig:
+                   expert_ff=0, shared_ff=0, share_every=2, moe_every=None, **kw) -> BozevikConfig:
     """n_layers latent-attention layers; every ``share_every``-th attends the previous owner's cache; with experts > 0
-    those layers route (the others are dense)."""
+    every ``moe_every``-th layer routes (default: the sharing layers), the others are dense."""
     layers, owner = [], 0
     for i in range(n_layers):
         shares = share_every > 0 and i % share_every == share_every - 1
@@ -235,7 +235,8 @@ def _bozevik_stack(name, vocab, width, n_layers, heads, dim, rot_dim, vdim, kv_r
             owner = i
         mix = LatentMixerSpec(heads, dim, rot_dim, vdim, kv_rank, q_rank, 10000.0, rot_dim, (dim + rot_dim) ** -0.5,
                               owner if shares else None)
-        if experts and shares:
+        routed = shares if moe_every is None else i % moe_every == moe_every - 1
+        if experts and routed:
             mlp = MoeSpec(experts, top, GluSpec(expert_ff, 7.0), GluSpec(shared_ff, 7.0) if shared_ff else None)
         else:
             mlp = GluSpec(ff, 7.0)

@@ -640,7 +640,10 @@ def rope_pairs(src, dst, positions, rope):
     return reference.rope_pairs(src, dst, positions, rope)
 
 
-LATENT_ATTN_PART = 256  # keys per split-KV partition of latent_attn's decode form (latent_attention.hip PART)
+def latent_attn_parts(rows: int, span: int, target_wgs: int = 512, min_tokens: int = 64) -> int:
+    """Split-KV partitions of a decode step's latent_attn: enough workgroups (rows x partitions) to fill the chip,
+    partitions of at least ``min_tokens`` keys.  ``span``: tokens the block table covers (the step's context bucket)."""
+    return max(1, min(-(-span // min_tokens), -(-target_wgs // max(1, rows)), 1024))
 
 
 LATENT_ATTN_IMPL = 1 if os.environ.get("SYMMETRY_LATENT_ATTN", "mfma") == "wave" else 0  # A/B: the all-shapes kernel
@@ -649,8 +652,9 @@ LATENT_ATTN_IMPL = 1 if os.environ.get("SYMMETRY_LATENT_ATTN", "mfma") == "wave"
 def latent_attn(q, cache, block_tables, row_seq, positions, scale, kv_rank, out, part_o=None, part_ml=None,
                 tiles=None, cu_q=None, impl=None):
     """Causal softmax attention of q [T, H, Dk] over the paged latent cache [NB, BS, Dk]: keys are whole cache rows,
-    values their first kv_rank entries; row r sees keys 0..positions[r] of sequence row_seq[r].  ``part_o`` /
-    ``part_ml``: split-KV scratch (decode steps: one partition per 256 keys, merged in a second launch).
+    values their first kv_rank entries; row r sees keys 0..positions[r] of sequence row_seq[r].  ``part_o``
+    [T, H, parts, kv_rank] / ``part_ml`` [T, H, parts, 2]: split-KV scratch (decode steps: ``parts`` equal partitions of
+    the block-table span, merged in a second launch; ``latent_attn_parts`` picks the count).
     ``tiles`` [n, 2] (sequence, first row of a 64-row tile within the sequence's run) + ``cu_q``: the prompt form of
     the MFMA kernel (bf16, Dk % 32 == 0, kv_rank % 16 == 0); without them that kernel takes one row per sequence
     (decode steps).  Other shapes, fp32 and ``impl=1`` run the one-wave-per-(row, head) kernel.  Returns the

@@ -66,6 +66,14 @@ def _cfg_c():
     ])
 
 
+def _cfg_d():
+    """Width 128 with 64-wide experts: bf16 on the GPU runs the expert products on the MFMA grouped GEMM."""
+    return O.make_config(width=128, vocab=160, eps=1e-5, logit_scale=1.2, layers=[
+        {"type": "latent_attention", "mixer": O.mixer(heads=4, dim=16, rot_dim=16, vdim=16, kv_rank=48, q_rank=32, base=1000.0, scale=0.2),
+         "mlp": O.moe(experts=6, top=2, ff=64, limit=1.5, shared_ff=128, shared_limit=2.0)},
+    ])
+
+
 def _checkpoint(tmp_path, cfg, seed=0, tensors=None):
     from safetensors.torch import save_file
 
@@ -124,7 +132,7 @@ def _oracle(cfg, tensors, ids):
 # ---- whole prompts, decoding, portions ----------------------------------------------------------------
 @pytest.mark.parametrize("device", DEVICES)
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("make", [_cfg_a, _cfg_b, _cfg_c])
+@pytest.mark.parametrize("make", [_cfg_a, _cfg_b, _cfg_c, _cfg_d])
 def test_prompt_decode_and_portions_agree_with_oracle(tmp_path, device, dtype, make):
     device = _device(device)
     cfg = make()
@@ -306,14 +314,13 @@ def test_latent_attn_mfma_forms_against_the_wave_kernel(H, r, rot):
         outs[name] = o.float().cpu()
         assert float((outs[name] - want).abs().max()) < 3e-2, name
     # split-KV partitions (decode form): rows of different sequences, context far past one partition
-    parts = -(-(mb * bs) // ops.LATENT_ATTN_PART)
     sel = torch.tensor([129, 130 + 69, 200, 201 + 63])                    # last rows of the four runs
-    for impl in (0, 1):
+    for impl, parts in ((0, 3), (1, 3), (0, 10), (1, 10), (0, 20)):
         o = torch.zeros(4, H, r, dtype=torch.bfloat16, device=dev)
         po = torch.zeros(4, H, parts, r, device=dev)
         pml = torch.zeros(4, H, parts, 2, device=dev)
         ops.latent_attn(d(q[sel]), d(cache), d(table), d(torch.arange(4).int()), d(pos[sel]), scale, r, o, po, pml, impl=impl)
-        assert float((o.float().cpu() - want[sel]).abs().max()) < 3e-2, impl
+        assert float((o.float().cpu() - want[sel]).abs().max()) < 3e-2, (impl, parts)
 
 
 # ---- each mechanism alone: op vs oracle function ------------------------------------------------------
