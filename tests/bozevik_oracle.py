@@ -12,6 +12,8 @@ import math
 import torch
 
 GLU_ALPHA = 1.702
+ROUTER_MARGINS = None  # a list: moe_ff appends, per call, the smallest gap between a token's last chosen and first
+                       # rejected router logit (tests use it to keep close calls out of reduced-precision comparisons)
 
 
 def rms_unit(x, eps):
@@ -81,8 +83,12 @@ def glu_ff(p, pre, h, limit):
 
 def moe_ff(p, pre, mlp, h):
     E, k = mlp["router"]["experts"], mlp["router"]["top"]
-    s = torch.sigmoid(h @ p[pre + "router"].T)
+    z = h @ p[pre + "router"].T
+    s = torch.sigmoid(z)
     top = s.topk(k, dim=-1)
+    if ROUTER_MARGINS is not None and k < E:
+        zs = z.sort(-1, descending=True).values
+        ROUTER_MARGINS.append(float((zs[:, k - 1] - zs[:, k]).min()))
     out = torch.zeros_like(h)
     for t in range(h.shape[0]):
         for j in range(k):

@@ -104,6 +104,21 @@ def _tokens(n, vocab, seed):
     return torch.randint(0, vocab, (n,), generator=g).tolist()
 
 
+def _clear_tokens(cfg, tensors, n, seed, margin=0.08):
+    """Token ids whose routing is no close call anywhere (every router's last chosen logit leads the first rejected
+    one by ``margin``): bf16 activations may resolve a near-tie the other way, which is no fault of the engine."""
+    for s in range(seed, seed + 200):
+        ids = _tokens(n, cfg["vocab"], s)
+        O.ROUTER_MARGINS = []
+        try:
+            O.forward(cfg, tensors, ids, torch.float64)
+            if all(m > margin for m in O.ROUTER_MARGINS):
+                return ids
+        finally:
+            O.ROUTER_MARGINS = None
+    raise AssertionError("no token sequence without a routing near-tie in 200 seeds")
+
+
 def _replay(eng, plan, requests):
     """plan: list of steps, each a list of (request name, token count).  Every position's logits are asked for.
     Returns {name: logits [len, V]}."""
@@ -138,7 +153,7 @@ def test_prompt_decode_and_portions_agree_with_oracle(tmp_path, device, dtype, m
     cfg = make()
     path, tensors = _checkpoint(tmp_path, cfg)
     eng = _engine(path, device, dtype)
-    ids = _tokens((3 if make is not _cfg_c else 9) * BS + 5, cfg["vocab"], 1)   # (_cfg_c: past one 64-row query tile)
+    ids = _clear_tokens(cfg, tensors, (3 if make is not _cfg_c else 9) * BS + 5, 1)   # (_cfg_c: past one 64-row query tile)
     want = _oracle(cfg, tensors, ids)
     n = len(ids)
     plans = {
@@ -165,7 +180,7 @@ def test_mixed_batches_reuse_of_blocks_and_slots(tmp_path, device, dtype):
     cfg = _cfg_a()
     path, tensors = _checkpoint(tmp_path, cfg, seed=3)
     eng = _engine(path, device, dtype, blocks=12)
-    reqs = {k: _tokens(n, cfg["vocab"], 10 + i) for i, (k, n) in
+    reqs = {k: _clear_tokens(cfg, tensors, n, 100 * i) for i, (k, n) in
             enumerate([("a", 1), ("b", 37), ("c", 2 * BS), ("d", 9), ("e", 50), ("f", BS + 1), ("g", 3)])}
     plan = [
         [("b", 20), ("a", 1), ("c", 2), ("d", 1)],
