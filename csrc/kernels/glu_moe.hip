@@ -41,7 +41,34 @@ __global__ __launch_bounds__(NT) void sigmoid_topk_kernel(const T* __restrict__ 
   for (int e = wave; e < E; e += NT / 64) {
     const T* wr = Wr + (long long)e * d;
     float s = 0.f;
-    for (int c = lane; c < d; c += 64) s += xs[c] * (float)wr[c];
+    if constexpr (sizeof(T) == 2) {
+      if ((d & 7) == 0) {
+        // 16-byte loads, four in flight per lane (a plain strided loop waits for every load in turn)
+        float acc[4] = {0.f, 0.f, 0.f, 0.f};
+        int c = lane * 8;
+        for (; c + 3 * 512 < d; c += 4 * 512) {
+          float f[4][8];
+#pragma unroll
+          for (int u = 0; u < 4; ++u) load8(reinterpret_cast<const bf16*>(wr) + c + u * 512, f[u]);
+#pragma unroll
+          for (int u = 0; u < 4; ++u)
+#pragma unroll
+            for (int i = 0; i < 8; ++i) acc[u] += xs[c + u * 512 + i] * f[u][i];
+        }
+        for (; c < d; c += 512) {
+          float f[8];
+          load8(reinterpret_cast<const bf16*>(wr) + c, f);
+#pragma unroll
+          for (int i = 0; i < 8; ++i) acc[0] += xs[c + i] * f[i];
+        }
+        s = (acc[0] + acc[1]) + (acc[2] + acc[3]);
+      } else {
+        for (int c = lane; c < d; c += 64) s += xs[c] * (float)wr[c];
+      }
+    } else {
+#pragma unroll 4
+      for (int c = lane; c < d; c += 64) s += xs[c] * (float)wr[c];
+    }
     s = wave_sum(s);
     if (lane == 0) score[e] = 1.f / (1.f + expf(-s));
   }
@@ -170,10 +197,14 @@ __global__ __launch_bounds__(NT) void grouped_linear_kernel(const T* __restrict_
 template <typename T>
 __global__ __launch_bounds__(NT) void gather_sum_kernel(const T* __restrict__ y, const int* __restrict__ dst, int k,
                                                         const T* __restrict__ extra, float* __restrict__ out, int d) {
+  __shared__ int rows[64];
   const int t = blockIdx.x;
+  for (int j = threadIdx.x; j < k && j < 64; j += NT) rows[j] = dst[t * k + j];
+  __syncthreads();
+#pragma unroll 4
   for (int c = threadIdx.x; c < d; c += NT) {
     float s = extra ? (float)extra[(long long)t * d + c] : 0.f;
-    for (int j = 0; j < k; ++j) s += (float)y[(long long)dst[t * k + j] * d + c];
+    for (int j = 0; j < k; ++j) s += (float)y[(long long)(j < 64 ? rows[j] : dst[t * k + j]) * d + c];
     out[(long long)t * d + c] = s;
   }
 }
