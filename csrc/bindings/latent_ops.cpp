@@ -202,6 +202,9 @@ int64_t latent_attn(const Tensor& q, const Tensor& cache, const Tensor& block_ta
   a.kv_rank = (int)kv_rank;
   a.BS = (int)cache.size(1);
   a.max_blocks = (int)block_tables.size(1);
+  a.bs_shift = -1;
+  for (int sh = 0; sh < 20; ++sh)
+    if ((1 << sh) == a.BS) a.bs_shift = sh;
   TORCH_CHECK(cache.size(2) == a.Dk && kv_rank > 0 && kv_rank <= a.Dk && kv_rank <= 512 && a.Dk <= 8192 &&
                   out.numel() == (int64_t)a.T * a.H * kv_rank && row_seq.numel() >= a.T && positions.numel() >= a.T &&
                   a.H <= 65535, "latent_attn: shapes");

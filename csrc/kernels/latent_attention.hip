@@ -239,14 +239,23 @@ __global__ __launch_bounds__(256) void latent_attn_merge_kernel(LatentAttnArgs a
 constexpr int KT = 32;        // keys per staged tile
 constexpr int LDV = KT + 4;   // row pitch (elements) of the transposed latent tile
 
-// NW waves per workgroup (4), 16 query vectors each.  Prompt form (DECODE = false): a tile of 64 rows of one head.
-// Decode form: one row, up to 64 of its heads, one key partition per workgroup.
+// NW waves per workgroup in QG = NW / DSPLIT groups of 16 query vectors; the DSPLIT waves of a group share the
+// query vectors (each computes the scores and the softmax, redundantly and identically) and split the latent dims
+// of the weighted sum, which divides the accumulator registers -- the bulk of a wave's registers at kv_rank 512 --
+// so that two waves fit a SIMD and one's LDS latency hides behind the other's MFMAs.
+// Prompt form (DECODE = false): a tile of 16 * QG rows of one head.  Decode form: one row, 16 * QG of its heads, one
+// key partition per workgroup (few heads: fewer groups, more dim splitting, so no wave idles).
 // The next tile's cache rows are fetched into registers while the current tile is multiplied (the global latency
 // hides behind the MFMAs); they go to LDS between two barriers at the top of the next iteration.
-template <int NKM, int RTM, bool DECODE, int NW>
+// EXACT: Dk == 32 * NKM and kv_rank == 16 * RTM, so the unrolled MFMA loops carry no bounds tests (a test on a
+// runtime count makes the compiler compute the MFMA anyway and select the accumulator afterwards: four selects,
+// through the accumulator registers, per MFMA).  The inexact instantiation serves every smaller tiled shape.
+template <int NKM, int RTM, bool DECODE, int NW, int DSPLIT, bool EXACT>
 __global__ __launch_bounds__(64 * NW) void latent_attn_mfma_kernel(LatentAttnArgs a) {
   extern __shared__ __attribute__((aligned(16))) char smem[];
   constexpr int NTH = 64 * NW;
+  constexpr int QG = NW / DSPLIT;                       // query-vector groups
+  constexpr int RTD = RTM / DSPLIT;                     // 16-dim output tiles per wave (upper bound)
   constexpr int CSTEP = NTH / 32;                       // 16-byte chunks of a row taken per pass of the workgroup
   constexpr int CHM = (NKM * 4 + CSTEP - 1) / CSTEP;    // passes (chunks per thread)
   // up to 9 passes stay in registers across the multiply (prefetch); workgroups of fewer waves have more passes per
@@ -254,20 +263,21 @@ __global__ __launch_bounds__(64 * NW) void latent_attn_mfma_kernel(LatentAttnArg
   constexpr bool PREFETCH = CHM <= 9;
   constexpr int NB = PREFETCH ? CHM : 9;
   const int Dk = a.Dk, r = a.kv_rank, H = a.H;
-  const int nk = Dk >> 5, rt = r >> 4, nchunk = Dk >> 3;
+  const int nk = EXACT ? NKM : Dk >> 5, rtd = EXACT ? RTD : (r >> 4) / DSPLIT, nchunk = EXACT ? NKM * 4 : Dk >> 3;
   const int ldk = Dk + 8;
   bf16* Ks = reinterpret_cast<bf16*>(smem);  // [KT][ldk] key-major cache rows
   bf16* Vt = Ks + KT * ldk;                   // [r][LDV] latent part, dim-major
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int n = lane & 15, g = lane >> 4;
+  const int qg = wave % QG, dh = wave / QG;             // this wave's query group and latent-dim share
   int seq, qrow, head, limit, k_lo, k_hi, wave_hi, wave_lo, part = 0;  // wave_lo: keys every query vector of the wave sees
   bool valid, wave_active;
   if constexpr (DECODE) {
     qrow = blockIdx.x;
     seq = a.row_seq[qrow];
-    head = blockIdx.y * 16 * NW + wave * 16 + n;
+    head = blockIdx.y * 16 * QG + qg * 16 + n;
     valid = head < H;
-    wave_active = blockIdx.y * 16 * NW + wave * 16 < H;
+    wave_active = blockIdx.y * 16 * QG + qg * 16 < H;
     limit = a.positions[qrow];
     part = blockIdx.z;
     k_lo = a.parts > 1 ? part * a.part_tokens : 0;
@@ -280,25 +290,25 @@ __global__ __launch_bounds__(64 * NW) void latent_attn_mfma_kernel(LatentAttnArg
     const int off = a.tiles[2 * blockIdx.x + 1];
     const int q0 = a.cu_q[seq], qlen = a.cu_q[seq + 1] - q0;
     if (off >= qlen) return;  // padding tile
-    const int rin = off + wave * 16 + n;
+    const int rin = off + qg * 16 + n;
     valid = rin < qlen;
-    wave_active = off + wave * 16 < qlen;
+    wave_active = off + qg * 16 < qlen;
     qrow = q0 + min(rin, qlen - 1);
     head = blockIdx.y;
     limit = a.positions[qrow];
     k_lo = 0;
-    k_hi = a.positions[q0 + min(off + 16 * NW - 1, qlen - 1)] + 1;       // a run's rows are consecutive positions
-    wave_hi = a.positions[q0 + min(off + wave * 16 + 15, qlen - 1)] + 1;
-    wave_lo = a.positions[q0 + min(off + wave * 16, qlen - 1)] + 1;
+    k_hi = a.positions[q0 + min(off + 16 * QG - 1, qlen - 1)] + 1;       // a run's rows are consecutive positions
+    wave_hi = a.positions[q0 + min(off + qg * 16 + 15, qlen - 1)] + 1;
+    wave_lo = a.positions[q0 + min(off + qg * 16, qlen - 1)] + 1;
   }
   const bf16* qp = (const bf16*)a.q + ((long long)qrow * H + min(head, H - 1)) * Dk;
   bf16x8 qf[NKM];
 #pragma unroll
   for (int s = 0; s < NKM; ++s)
-    if (s < nk) qf[s] = *reinterpret_cast<const bf16x8*>(qp + s * 32 + g * 8);
-  f32x4 o[RTM];
+    if (EXACT || s < nk) qf[s] = *reinterpret_cast<const bf16x8*>(qp + s * 32 + g * 8);
+  f32x4 o[RTD];  // output tile dt of this wave covers dims (dh * rtd + dt) * 16 ..
 #pragma unroll
-  for (int i = 0; i < RTM; ++i) o[i] = f32x4{0.f, 0.f, 0.f, 0.f};
+  for (int i = 0; i < RTD; ++i) o[i] = f32x4{0.f, 0.f, 0.f, 0.f};
   float m = -INFINITY, l = 0.f;
   const int* bt = a.block_tables + (long long)seq * a.max_blocks;
   const bf16* cache = (const bf16*)a.cache;
@@ -306,7 +316,8 @@ __global__ __launch_bounds__(64 * NW) void latent_attn_mfma_kernel(LatentAttnArg
   uint4 pre[NB];
   auto fetch = [&](int k0, int i0) {
     const int key = min(k0 + key_in, k_hi - 1);
-    const bf16* src = cache + ((long long)bt[key / a.BS] * a.BS + key % a.BS) * Dk;
+    const int blk = a.bs_shift >= 0 ? key >> a.bs_shift : key / a.BS;  // (no integer divide for power-of-two blocks)
+    const bf16* src = cache + ((long long)bt[blk] * a.BS + (key - blk * a.BS)) * Dk;
 #pragma unroll
     for (int i = 0; i < NB; ++i) {
       const int c = c0 + (i0 + i) * CSTEP;
@@ -353,7 +364,7 @@ __global__ __launch_bounds__(64 * NW) void latent_attn_mfma_kernel(LatentAttnArg
       const bf16* kr = Ks + n * ldk + g * 8;
 #pragma unroll
       for (int s = 0; s < NKM; ++s)
-        if (s < nk) {
+        if (EXACT || s < nk) {
           acc[s & 1] = mfma16(*reinterpret_cast<const bf16x8*>(kr + s * 32), qf[s], acc[s & 1]);
           acc[2 + (s & 1)] = mfma16(*reinterpret_cast<const bf16x8*>(kr + 16 * ldk + s * 32), qf[s], acc[2 + (s & 1)]);
         }
@@ -385,8 +396,8 @@ __global__ __launch_bounds__(64 * NW) void latent_attn_mfma_kernel(LatentAttnArg
       const float alpha = __expf(m - m_new);
       l *= alpha;
 #pragma unroll
-      for (int dt = 0; dt < RTM; ++dt)
-        if (dt < rt) o[dt] = o[dt] * alpha;
+      for (int dt = 0; dt < RTD; ++dt)
+        if (EXACT || dt < rtd) o[dt] = o[dt] * alpha;
       m = m_new;
     }
     float ps = 0.f;
@@ -403,10 +414,10 @@ __global__ __launch_bounds__(64 * NW) void latent_attn_mfma_kernel(LatentAttnArg
     ps += __shfl_xor(ps, 32, 64);
     l += ps;
     // O^T += V^T P^T: k index g * 8 + j of the product is key g * 4 + j (j < 4) / 16 + g * 4 + j - 4 of the tile
-    const bf16* vr = Vt + n * LDV + g * 4;
+    const bf16* vr = Vt + (dh * rtd * 16 + n) * LDV + g * 4;
 #pragma unroll
-    for (int dt = 0; dt < RTM; ++dt)
-      if (dt < rt) {
+    for (int dt = 0; dt < RTD; ++dt)
+      if (EXACT || dt < rtd) {
         Pack8 va;
         const uint2 lo = *reinterpret_cast<const uint2*>(vr + dt * 16 * LDV);
         const uint2 hi = *reinterpret_cast<const uint2*>(vr + dt * 16 * LDV + 16);
@@ -415,13 +426,13 @@ __global__ __launch_bounds__(64 * NW) void latent_attn_mfma_kernel(LatentAttnArg
       }
   }
   if (!valid) return;
-  // o[dt][i]: dim dt * 16 + g * 4 + i of query vector n
+  // o[dt][i]: dim (dh * rtd + dt) * 16 + g * 4 + i of query vector n
   if (a.parts == 1) {
-    bf16* out = (bf16*)a.out + ((long long)qrow * H + head) * r;
+    bf16* out = (bf16*)a.out + ((long long)qrow * H + head) * r + dh * rtd * 16;
     const float inv = 1.f / l;
 #pragma unroll
-    for (int dt = 0; dt < RTM; ++dt)
-      if (dt < rt) {
+    for (int dt = 0; dt < RTD; ++dt)
+      if (EXACT || dt < rtd) {
         bf16x4 v;
 #pragma unroll
         for (int i = 0; i < 4; ++i) v[i] = (bf16)(o[dt][i] * inv);
@@ -429,44 +440,53 @@ __global__ __launch_bounds__(64 * NW) void latent_attn_mfma_kernel(LatentAttnArg
       }
   } else {
     const long long pi = ((long long)qrow * H + head) * a.parts + part;
-    float* po = a.part_o + pi * r;
+    float* po = a.part_o + pi * r + dh * rtd * 16;
 #pragma unroll
-    for (int dt = 0; dt < RTM; ++dt)
-      if (dt < rt) *reinterpret_cast<f32x4*>(po + dt * 16 + g * 4) = o[dt];
-    if (g == 0) {
+    for (int dt = 0; dt < RTD; ++dt)
+      if (EXACT || dt < rtd) *reinterpret_cast<f32x4*>(po + dt * 16 + g * 4) = o[dt];
+    if (g == 0 && dh == 0) {
       a.part_ml[2 * pi] = m;
       a.part_ml[2 * pi + 1] = l;
     }
   }
 }
 
-template <int NKM, int RTM, bool DECODE, int NW>
+template <int NKM, int RTM, bool DECODE, int NW, int DSPLIT, bool EXACT>
 void mfma_launch_one(const LatentAttnArgs& a, dim3 grid, hipStream_t s) {
   const size_t lds = ((size_t)KT * (a.Dk + 8) + (size_t)a.kv_rank * LDV) * sizeof(bf16);
   static bool raised = false;  // (per instantiation) dynamic LDS beyond the 64 KB default
   if (!raised) {
-    hipFuncSetAttribute(reinterpret_cast<const void*>(&latent_attn_mfma_kernel<NKM, RTM, DECODE, NW>),
+    hipFuncSetAttribute(reinterpret_cast<const void*>(&latent_attn_mfma_kernel<NKM, RTM, DECODE, NW, DSPLIT, EXACT>),
                         hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024);
     raised = true;
   }
-  latent_attn_mfma_kernel<NKM, RTM, DECODE, NW><<<grid, 64 * NW, lds, s>>>(a);
+  latent_attn_mfma_kernel<NKM, RTM, DECODE, NW, DSPLIT, EXACT><<<grid, 64 * NW, lds, s>>>(a);
 }
 
-template <int NKM, int RTM>
+template <int NKM, int RTM, bool EXACT>
 void mfma_launch(const LatentAttnArgs& a, hipStream_t s) {
-  // four waves in both forms.  Decode rows of fewer than 64 heads leave waves without query vectors; those still
-  // stage, so every thread holds one tile's share in registers and the next tile is prefetched across the multiply
-  // (one- and two-wave workgroups measured slower: 8 x 1024 tokens, 16 heads 41.9 vs 31.5 us)
-  if (a.tiles) mfma_launch_one<NKM, RTM, false, 4>(a, dim3(a.ntiles, a.H), s);
-  else mfma_launch_one<NKM, RTM, true, 4>(a, dim3(a.T, (a.H + 63) / 64, a.parts), s);
+  const int rt = a.kv_rank / 16;
+  if (a.tiles) {
+    // 64 rows of one head; eight waves (each row group twice, half the latent dims each) where the dims split
+    // (8 x 1024 tokens, 16 heads, kv_rank 512: 1090 -> 900 us)
+    if (rt % 2 == 0) mfma_launch_one<NKM, RTM, false, 8, 2, EXACT>(a, dim3(a.ntiles, a.H), s);
+    else mfma_launch_one<NKM, RTM, false, 4, 1, false>(a, dim3(a.ntiles, a.H), s);
+    return;
+  }
+  // decode rows.  Up to 16 heads: one query group computes, the other three waves only stage (splitting the dims
+  // over them re-reads the key tile four times: 64 x 2048 tokens 119 vs 104 us); up to 32 heads: two groups x two
+  // dim halves; more: four groups x two (eight waves).  Odd tile counts fall back to unsplit dims.
+  if (a.H <= 16 || rt % 2) mfma_launch_one<NKM, RTM, true, 4, 1, EXACT>(a, dim3(a.T, (a.H + 63) / 64, a.parts), s);
+  else if (a.H <= 32) mfma_launch_one<NKM, RTM, true, 4, 2, EXACT>(a, dim3(a.T, (a.H + 31) / 32, a.parts), s);
+  else mfma_launch_one<NKM, RTM, true, 8, 2, EXACT>(a, dim3(a.T, (a.H + 63) / 64, a.parts), s);
 }
 
 bool mfma_dispatch(const LatentAttnArgs& a, hipStream_t s) {
   const int nk = a.Dk / 32, rt = a.kv_rank / 16;
   if (a.Dk % 32 || a.kv_rank % 16 || nk > 18 || rt > 32 || a.part_tokens % KT) return false;
-  if (nk <= 5 && rt <= 8) mfma_launch<5, 8>(a, s);
-  else if (nk <= 10 && rt <= 16) mfma_launch<10, 16>(a, s);
-  else mfma_launch<18, 32>(a, s);
+  if (nk == 18 && rt == 32) mfma_launch<18, 32, true>(a, s);       // 512 + 64
+  else if (nk == 5 && rt == 8) mfma_launch<5, 8, true>(a, s);      // 128 + 32
+  else mfma_launch<18, 32, false>(a, s);                           // every other tiled shape
   return true;
 }
 

@@ -52,6 +52,7 @@ struct LatentAttnArgs {
   float* part_o;        // split-KV partials (decode form): [T][H][parts][kv_rank], [T][H][parts][2]
   float* part_ml;
   int T, H, Dk, kv_rank, BS, max_blocks;
+  int bs_shift;            // log2(BS), or -1 if BS is no power of two
   int parts, part_tokens;  // split-KV: partition p of a row covers keys [p * part_tokens, (p + 1) * part_tokens)
   float scale;
   // prompt form of the MFMA kernel: 64-row query tiles (sequence, first row within the sequence's run) over the
