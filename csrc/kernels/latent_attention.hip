@@ -353,11 +353,32 @@ __global__ __launch_bounds__(64 * NW) void latent_attn_mfma_kernel(LatentAttnArg
     __syncthreads();
     if constexpr (PREFETCH)
       if (k0 + KT < k_hi) fetch(k0 + KT, 0);
-    if (!wave_active || k0 >= wave_hi) continue;
     // S^T: rows = keys (sub * 16 + g * 4 + i), column = this lane's query vector n
-    // (four independent accumulator chains: both 16-key subtiles, even and odd k steps)
+    const bool active = wave_active && k0 < wave_hi;  // (the same for the waves that share a query group)
     f32x4 st[2];
-    {
+    if constexpr (DSPLIT == 2) {
+      // the two waves of a query group each score one 16-key subtile (four accumulator chains over the k steps) and
+      // swap the results through LDS: half the score MFMAs and key-tile reads of computing both subtiles twice
+      f32x4* xch = reinterpret_cast<f32x4*>(Vt + r * LDV);  // [QG][2][64]
+      f32x4 mine = {0.f, 0.f, 0.f, 0.f};
+      if (active) {
+        f32x4 acc[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) acc[i] = f32x4{0.f, 0.f, 0.f, 0.f};
+        const bf16* kr = Ks + (dh * 16 + n) * ldk + g * 8;
+#pragma unroll
+        for (int s = 0; s < NKM; ++s)
+          if (EXACT || s < nk) acc[s & 3] = mfma16(*reinterpret_cast<const bf16x8*>(kr + s * 32), qf[s], acc[s & 3]);
+        mine = (acc[0] + acc[1]) + (acc[2] + acc[3]);
+        xch[(qg * 2 + dh) * 64 + lane] = mine;
+      }
+      __syncthreads();
+      if (!active) continue;
+      st[0] = mine;                                         // (own subtile first; put in key order below)
+      st[1] = xch[(qg * 2 + 1 - dh) * 64 + lane];
+    } else {
+      if (!active) continue;
+      // (four independent accumulator chains: both 16-key subtiles, even and odd k steps)
       f32x4 acc[4];
 #pragma unroll
       for (int i = 0; i < 4; ++i) acc[i] = f32x4{0.f, 0.f, 0.f, 0.f};
@@ -370,6 +391,13 @@ __global__ __launch_bounds__(64 * NW) void latent_attn_mfma_kernel(LatentAttnArg
         }
       st[0] = acc[0] + acc[1];
       st[1] = acc[2] + acc[3];
+    }
+    if constexpr (DSPLIT == 2) {
+      if (dh) {  // st[] indexed by a runtime dh above: keep it in registers
+        const f32x4 t = st[0];
+        st[0] = st[1];
+        st[1] = t;
+      }
     }
     // scale; mask only where a tile reaches past some query vector's last key (the diagonal tiles, the range's tail)
     const bool edge = k0 + KT > wave_lo || k0 + KT > k_hi;  // wave-uniform
@@ -453,7 +481,8 @@ __global__ __launch_bounds__(64 * NW) void latent_attn_mfma_kernel(LatentAttnArg
 
 template <int NKM, int RTM, bool DECODE, int NW, int DSPLIT, bool EXACT>
 void mfma_launch_one(const LatentAttnArgs& a, dim3 grid, hipStream_t s) {
-  const size_t lds = ((size_t)KT * (a.Dk + 8) + (size_t)a.kv_rank * LDV) * sizeof(bf16);
+  const size_t lds = ((size_t)KT * (a.Dk + 8) + (size_t)a.kv_rank * LDV) * sizeof(bf16) +
+                     (DSPLIT == 2 ? (NW / 2) * 2 * 64 * sizeof(f32x4) : 0);  // + the score exchange of the wave pairs
   static bool raised = false;  // (per instantiation) dynamic LDS beyond the 64 KB default
   if (!raised) {
     hipFuncSetAttribute(reinterpret_cast<const void*>(&latent_attn_mfma_kernel<NKM, RTM, DECODE, NW, DSPLIT, EXACT>),
