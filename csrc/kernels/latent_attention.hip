@@ -513,8 +513,7 @@ void mfma_launch(const LatentAttnArgs& a, hipStream_t s) {
 bool mfma_dispatch(const LatentAttnArgs& a, hipStream_t s) {
   const int nk = a.Dk / 32, rt = a.kv_rank / 16;
   if (a.Dk % 32 || a.kv_rank % 16 || nk > 18 || rt > 32 || a.part_tokens % KT) return false;
-  if (nk == 18 && rt == 32) mfma_launch<18, 32, true>(a, s);       // 512 + 64
-  else if (nk == 5 && rt == 8) mfma_launch<5, 8, true>(a, s);      // 128 + 32
+  if (nk == 18 && rt == 32) mfma_launch<18, 32, true>(a, s);       // latent 512 + rotary 64
   else mfma_launch<18, 32, false>(a, s);                           // every other tiled shape
   return true;
 }
