@@ -335,6 +335,8 @@ class LLMEngine:
         given = []
         with self.lock:
             for rid, tokens, want in entries:
+                if not tokens:
+                    continue
                 ent = self.requests.get(rid)
                 if ent is None:
                     seq = Sequence(rid, [], SamplingParams(max_tokens=1), eos_ids=())

@@ -46,26 +46,24 @@ GLU_ALPHA = 1.702  # slope of the gate's sigmoid (fixed by the design)
 class LatentKVCache:
     """Paged latent cache + per-sequence carried state.
 
-    ``kv`` [planes, NB, BS, r + rot]: one plane per layer that owns a down-projection (layers that attend another
-    layer's latents have none), a row = normalised latent | rotated shared key part.  Zero-initialised: every byte
-    is finite, so rows of padded batch entries (block 0) contribute finite scores.
+    ``kv``: one plane [NB, BS, r + rot] per layer that owns a down-projection (layers that attend another layer's
+    latents have none), a row = normalised latent | rotated shared key part; planes may differ in width (every
+    layer names its own sizes) and share the block numbering, so one BlockManager and one block table serve all.
+    Zero-initialised: every byte is finite, so rows of padded batch entries (block 0) contribute finite scores.
     ``state`` [slots, L, d] fp32: per live sequence and layer, the layer input row of the sequence's newest token
     (what the next step's token shift reads as x_prev).  Slots are handed out by the scheduler's StateSlotManager.
     """
 
     def __init__(self, cfg: BozevikConfig, num_blocks: int, block_size: int, num_slots: int, device, dtype):
         owners = cfg.cache_layers()
-        widths = {cfg.layers[i].mixer.kv_rank + cfg.layers[i].mixer.rot_dim for i in owners}
-        if len(widths) != 1:
-            raise NotImplementedError(f"cache planes of different widths {sorted(widths)} (one pool per width)")
-        self.width = widths.pop()
         self.plane = {layer: p for p, layer in enumerate(owners)}
         self.num_layers, self.num_blocks, self.block_size = cfg.num_layers, num_blocks, block_size
-        self.kv = torch.zeros(len(owners), num_blocks, block_size, self.width, device=device, dtype=dtype)
+        self.kv = [torch.zeros(num_blocks, block_size, cfg.layers[i].mixer.kv_rank + cfg.layers[i].mixer.rot_dim,
+                               device=device, dtype=dtype) for i in owners]
         self.state = torch.zeros(num_slots, cfg.num_layers, cfg.hidden_size, device=device, dtype=torch.float32)
 
     def nbytes(self) -> int:
-        return self.kv.numel() * self.kv.element_size() + self.state.numel() * 4
+        return sum(t.numel() * t.element_size() for t in self.kv) + self.state.numel() * 4
 
 
 class BozevikLM:

@@ -47,12 +47,15 @@ def _cfg_a():
 
 
 def _cfg_b():
-    """One layer of each feed-forward kind, odd sizes (nothing a multiple of 8 but the rotary), top 1."""
+    """One layer of each feed-forward kind, odd sizes (nothing a multiple of 8 but the rotary), top 1; a third layer
+    with a cache row of another width, rotary base and length than the first."""
     return O.make_config(width=50, vocab=77, eps=1e-6, logit_scale=1.0, layers=[
         {"type": "latent_attention", "mixer": O.mixer(heads=1, dim=10, rot_dim=6, vdim=14, kv_rank=70, q_rank=18, base=300.0, scale=0.4),
          "mlp": O.moe(experts=4, top=1, ff=22, limit=1.5, shared_ff=26, shared_limit=0.5)},
         {"type": "latent_attention", "mixer": O.mixer(heads=5, dim=6, rot_dim=6, vdim=6, kv_rank=70, q_rank=30, base=300.0, scale=0.35, kv_from=0),
          "mlp": O.dense(ff=33, limit=2.0)},
+        {"type": "latent_attention", "mixer": O.mixer(heads=2, dim=4, rot_dim=10, vdim=9, kv_rank=22, q_rank=12, base=90.0, scale=0.5),
+         "mlp": O.dense(ff=20, limit=1.0)},
     ])
 
 
