@@ -28,6 +28,26 @@ __global__ __launch_bounds__(NT) void clamped_glu_kernel(const T* __restrict__ g
   out[i] = (T)(g / (1.f + expf(-alpha * g)) * (u + 1.f));
 }
 
+// bf16, F % 8 == 0: eight columns per thread, 16-byte loads and stores (prompt-sized launches are bandwidth-bound)
+__global__ __launch_bounds__(NT) void clamped_glu_vec_kernel(const bf16* __restrict__ gu, bf16* __restrict__ out,
+                                                             long long nvec, int F, float limit, float alpha) {
+  const long long i = (long long)blockIdx.x * NT + threadIdx.x;
+  if (i >= nvec) return;
+  const int fv = F >> 3;
+  const long long r = i / fv;
+  const int c = (int)(i - r * fv) * 8;
+  float g[8], u[8], y[8];
+  load8(gu + r * 2 * F + c, g);
+  load8(gu + r * 2 * F + F + c, u);
+#pragma unroll
+  for (int j = 0; j < 8; ++j) {
+    const float gj = fminf(g[j], limit);
+    const float uj = fminf(fmaxf(u[j], -limit), limit);
+    y[j] = gj / (1.f + __expf(-alpha * gj)) * (uj + 1.f);
+  }
+  store8(out + r * F + c, y);
+}
+
 constexpr int MAX_EXPERTS = 1024;
 
 template <typename T>
@@ -214,6 +234,12 @@ __global__ __launch_bounds__(NT) void gather_sum_kernel(const T* __restrict__ y,
 void launch_clamped_glu(const void* gu, void* out, int R, int F, float limit, float alpha, int f32, hipStream_t s) {
   const long long n = (long long)R * F;
   if (n <= 0) return;
+  if (!f32 && F % 8 == 0) {
+    const long long nvec = n / 8;
+    clamped_glu_vec_kernel<<<(unsigned)((nvec + NT - 1) / NT), NT, 0, s>>>((const bf16*)gu, (bf16*)out, nvec, F, limit,
+                                                                         alpha);
+    return;
+  }
   const unsigned grid = (unsigned)((n + NT - 1) / NT);
   if (f32) clamped_glu_kernel<float><<<grid, NT, 0, s>>>((const float*)gu, (float*)out, n, F, limit, alpha);
   else clamped_glu_kernel<bf16><<<grid, NT, 0, s>>>((const bf16*)gu, (bf16*)out, n, F, limit, alpha);

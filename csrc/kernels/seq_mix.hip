@@ -117,6 +117,91 @@ __global__ __launch_bounds__(NT) void add_layer_norm_kernel(const TD* __restrict
   }
 }
 
+// Four consecutive columns per thread and pass (d % 4 == 0, d <= NT * 4 * G): 8- / 16-byte accesses for the
+// bandwidth-bound prompt-sized launches; the same arithmetic in the same order per element as the scalar kernel.
+template <typename V>
+SYM_DEV void ld4(const V* p, float* f);
+template <>
+SYM_DEV void ld4<float>(const float* p, float* f) {
+  const float4 v = *reinterpret_cast<const float4*>(p);
+  f[0] = v.x; f[1] = v.y; f[2] = v.z; f[3] = v.w;
+}
+template <>
+SYM_DEV void ld4<bf16>(const bf16* p, float* f) {
+  const bf16x4 v = *reinterpret_cast<const bf16x4*>(p);
+#pragma unroll
+  for (int i = 0; i < 4; ++i) f[i] = (float)v[i];
+}
+SYM_DEV void st4(float* p, const float* f) { *reinterpret_cast<float4*>(p) = make_float4(f[0], f[1], f[2], f[3]); }
+SYM_DEV void st4(bf16* p, const float* f) {
+  bf16x4 v;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) v[i] = (bf16)f[i];
+  *reinterpret_cast<bf16x4*>(p) = v;
+}
+
+template <typename T, typename TD, int G>
+__global__ __launch_bounds__(NT) void add_layer_norm_vec_kernel(const TD* __restrict__ delta, const T* __restrict__ w,
+                                                                float eps, float* __restrict__ x,
+                                                                const int* __restrict__ save, float* __restrict__ state,
+                                                                long long state_stride, float* __restrict__ hist,
+                                                                long long hist_stride, const float* __restrict__ coef,
+                                                                int hist_idx, T* __restrict__ out_act, int d) {
+  __shared__ float scratch[NT / 64];
+  const int row = blockIdx.x;
+  const long long rb = (long long)row * d;
+  float dv[G][4], xv[G][4], wv[G][4];
+  float sum = 0.f;
+#pragma unroll
+  for (int i = 0; i < G; ++i) {
+    const int c = (threadIdx.x + i * NT) * 4;
+    if (c < d) {
+      ld4<TD>(delta + rb + c, dv[i]);
+      ld4<float>(x + rb + c, xv[i]);
+      ld4<T>(w + c, wv[i]);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) sum += dv[i][j];
+    }
+  }
+  const float mean = block_sum<NT>(sum, scratch) / (float)d;
+  float sq = 0.f;
+#pragma unroll
+  for (int i = 0; i < G; ++i)
+    if ((threadIdx.x + i * NT) * 4 < d) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const float v = dv[i][j] - mean;
+        sq += v * v;
+      }
+    }
+  const float rstd = 1.f / sqrtf(block_sum<NT>(sq, scratch) / (float)d + eps);
+  const int sv = save ? save[row] : -1;
+#pragma unroll
+  for (int i = 0; i < G; ++i) {
+    const int c = (threadIdx.x + i * NT) * 4;
+    if (c >= d) continue;
+    if (sv >= 0) st4(state + (long long)sv * state_stride + c, xv[i]);
+    float xn[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) xn[j] = xv[i][j] + (dv[i][j] - mean) * rstd * wv[i][j];
+    if (hist) {
+      st4(hist + (long long)hist_idx * hist_stride + rb + c, xn);
+      const float ci = coef[hist_idx];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) xn[j] *= ci;
+      for (int k = 0; k < hist_idx; ++k) {
+        float hv[4];
+        ld4<float>(hist + (long long)k * hist_stride + rb + c, hv);
+        const float ck = coef[k];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) xn[j] += ck * hv[j];
+      }
+    }
+    st4(x + rb + c, xn);
+    if (out_act) st4(out_act + rb + c, xn);
+  }
+}
+
 template <typename T>
 __global__ __launch_bounds__(NT) void layer_norm_kernel(const float* __restrict__ x, const long long* __restrict__ rows,
                                                         const T* __restrict__ w, float eps, T* __restrict__ out, int d) {
@@ -162,12 +247,22 @@ void add_layer_norm_pick(const void* delta, const void* w, float eps, float* x, 
 #define SYM_ALN(EPT)                                                                                                   \
   add_layer_norm_kernel<T, TD, EPT><<<T_, NT, 0, s>>>((const TD*)delta, (const T*)w, eps, x, save, state, state_stride, \
                                                       hist, hist_stride, coef, hist_idx, (T*)out_act, d)
+#define SYM_ALNV(G)                                                                                                   \
+  add_layer_norm_vec_kernel<T, TD, G><<<T_, NT, 0, s>>>((const TD*)delta, (const T*)w, eps, x, save, state,            \
+                                                        state_stride, hist, hist_stride, coef, hist_idx, (T*)out_act, d)
+  if (d % 4 == 0 && state_stride % 4 == 0 && d <= NT * 32) {
+    if (d <= NT * 8) SYM_ALNV(2);
+    else if (d <= NT * 16) SYM_ALNV(4);
+    else SYM_ALNV(8);
+    return;
+  }
   if (d <= NT * 4) SYM_ALN(4);
   else if (d <= NT * 8) SYM_ALN(8);
   else if (d <= NT * 16) SYM_ALN(16);
   else if (d <= NT * 32) SYM_ALN(32);
   else SYM_ALN(0);
 #undef SYM_ALN
+#undef SYM_ALNV
 }
 
 void launch_add_layer_norm(const void* delta, int delta_f32, const void* w, float eps, float* x, const int* save,
