@@ -219,7 +219,7 @@ __global__ __launch_bounds__(256) void latent_attn_merge_kernel(LatentAttnArgs a
   __syncthreads();
   const float inv = 1.f / (stat[4] + stat[5] + stat[6] + stat[7]);
   float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-#pragma unroll 2
+#pragma unroll 4
   for (int p = wave; p < np; p += 4) {
     const float* po = a.part_o + (p0 + p) * a.kv_rank;
     const float w = wp[p];
@@ -351,6 +351,7 @@ __global__ __launch_bounds__(64 * NW) void latent_attn_mfma_kernel(LatentAttnArg
       }
     }
     __syncthreads();
+    // (issued after the barrier: issuing it before, right behind the stash, measured 4 % slower)
     if constexpr (PREFETCH)
       if (k0 + KT < k_hi) fetch(k0 + KT, 0);
     // S^T: rows = keys (sub * 16 + g * 4 + i), column = this lane's query vector n
