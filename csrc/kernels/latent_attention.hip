@@ -260,13 +260,15 @@ __global__ __launch_bounds__(64 * NW) void latent_attn_mfma_kernel(LatentAttnArg
   constexpr int CHM = (NKM * 4 + CSTEP - 1) / CSTEP;    // passes (chunks per thread)
   // up to 9 passes stay in registers across the multiply (prefetch); workgroups of fewer waves have more passes per
   // thread than registers to spare and stage in batches instead (no prefetch: they run one or two tiles)
-  constexpr bool PREFETCH = CHM <= 9;
-  constexpr int NB = PREFETCH ? CHM : 9;
+  static_assert(CHM <= 9, "a thread keeps one tile's share of cache rows in registers");
+  constexpr int NB = CHM;
   const int Dk = a.Dk, r = a.kv_rank, H = a.H;
   const int nk = EXACT ? NKM : Dk >> 5, rtd = EXACT ? RTD : (r >> 4) / DSPLIT, nchunk = EXACT ? NKM * 4 : Dk >> 3;
   const int ldk = Dk + 8;
-  bf16* Ks = reinterpret_cast<bf16*>(smem);  // [KT][ldk] key-major cache rows
-  bf16* Vt = Ks + KT * ldk;                   // [r][LDV] latent part, dim-major
+  // two LDS stages, each [KT][ldk] key-major cache rows + [r][LDV] latent part dim-major; tile t lives in stage
+  // t & 1, so tile t + 1 is written while tile t is still being multiplied
+  const int stage_elems = KT * ldk + r * LDV;
+  bf16* const stage0 = reinterpret_cast<bf16*>(smem);
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int n = lane & 15, g = lane >> 4;
   const int qg = wave % QG, dh = wave / QG;             // this wave's query group and latent-dim share
@@ -324,7 +326,8 @@ __global__ __launch_bounds__(64 * NW) void latent_attn_mfma_kernel(LatentAttnArg
       if (c < nchunk) pre[i] = *reinterpret_cast<const uint4*>(src + c * 8);
     }
   };
-  auto stash = [&](int i0) {
+  auto stash = [&](int i0, bf16* Ks) {
+    bf16* Vt = Ks + KT * ldk;
 #pragma unroll
     for (int i = 0; i < NB; ++i) {
       const int c = c0 + (i0 + i) * CSTEP;
@@ -339,28 +342,29 @@ __global__ __launch_bounds__(64 * NW) void latent_attn_mfma_kernel(LatentAttnArg
       }
     }
   };
-  if constexpr (PREFETCH) fetch(k_lo, 0);
-  for (int k0 = k_lo; k0 < k_hi; k0 += KT) {
-    __syncthreads();  // the previous tile's fragment reads are done
-    if constexpr (PREFETCH) {
-      stash(0);
-    } else {
-      for (int i0 = 0; i0 < CHM; i0 += NB) {
-        fetch(k0, i0);
-        stash(i0);
-      }
+  // Per tile: barrier A (everyone is done with the previous tile's value product and score exchange, so the other
+  // stage and the exchange area may be overwritten; the stage written during the previous tile is visible) and, where
+  // wave pairs exchange scores, barrier B (this tile's exchanged scores are visible).  The global fetch of tile t + 2 is issued right after tile t + 1 went to LDS and has a whole
+  // tile of work to land.
+  fetch(k_lo, 0);
+  stash(0, stage0);
+  if (k_lo + KT < k_hi) fetch(k_lo + KT, 0);
+  int cur = 0;
+  for (int k0 = k_lo; k0 < k_hi; k0 += KT, cur ^= 1) {
+    const bf16* Ks = stage0 + cur * stage_elems;
+    const bf16* Vt = Ks + KT * ldk;
+    __syncthreads();  // A
+    if (k0 + KT < k_hi) {
+      stash(0, stage0 + (cur ^ 1) * stage_elems);
+      if (k0 + 2 * KT < k_hi) fetch(k0 + 2 * KT, 0);
     }
-    __syncthreads();
-    // (issued after the barrier: issuing it before, right behind the stash, measured 4 % slower)
-    if constexpr (PREFETCH)
-      if (k0 + KT < k_hi) fetch(k0 + KT, 0);
     // S^T: rows = keys (sub * 16 + g * 4 + i), column = this lane's query vector n
     const bool active = wave_active && k0 < wave_hi;  // (the same for the waves that share a query group)
     f32x4 st[2];
     if constexpr (DSPLIT == 2) {
       // the two waves of a query group each score one 16-key subtile (four accumulator chains over the k steps) and
       // swap the results through LDS: half the score MFMAs and key-tile reads of computing both subtiles twice
-      f32x4* xch = reinterpret_cast<f32x4*>(Vt + r * LDV);  // [QG][2][64]
+      f32x4* xch = reinterpret_cast<f32x4*>(stage0 + 2 * stage_elems);  // [QG][2][64]
       f32x4 mine = {0.f, 0.f, 0.f, 0.f};
       if (active) {
         f32x4 acc[4];
@@ -373,12 +377,12 @@ __global__ __launch_bounds__(64 * NW) void latent_attn_mfma_kernel(LatentAttnArg
         mine = (acc[0] + acc[1]) + (acc[2] + acc[3]);
         xch[(qg * 2 + dh) * 64 + lane] = mine;
       }
-      __syncthreads();
+      __syncthreads();  // B
       if (!active) continue;
       st[0] = mine;                                         // (own subtile first; put in key order below)
       st[1] = xch[(qg * 2 + 1 - dh) * 64 + lane];
     } else {
-      if (!active) continue;
+      if (!active) continue;  // (no exchange: barrier A alone orders the stages)
       // (four independent accumulator chains: both 16-key subtiles, even and odd k steps)
       f32x4 acc[4];
 #pragma unroll
@@ -482,12 +486,12 @@ __global__ __launch_bounds__(64 * NW) void latent_attn_mfma_kernel(LatentAttnArg
 
 template <int NKM, int RTM, bool DECODE, int NW, int DSPLIT, bool EXACT>
 void mfma_launch_one(const LatentAttnArgs& a, dim3 grid, hipStream_t s) {
-  const size_t lds = ((size_t)KT * (a.Dk + 8) + (size_t)a.kv_rank * LDV) * sizeof(bf16) +
+  const size_t lds = 2 * ((size_t)KT * (a.Dk + 8) + (size_t)a.kv_rank * LDV) * sizeof(bf16) +  // two stages
                      (DSPLIT == 2 ? (NW / 2) * 2 * 64 * sizeof(f32x4) : 0);  // + the score exchange of the wave pairs
   static bool raised = false;  // (per instantiation) dynamic LDS beyond the 64 KB default
   if (!raised) {
     hipFuncSetAttribute(reinterpret_cast<const void*>(&latent_attn_mfma_kernel<NKM, RTM, DECODE, NW, DSPLIT, EXACT>),
-                        hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024);
+                        hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
     raised = true;
   }
   latent_attn_mfma_kernel<NKM, RTM, DECODE, NW, DSPLIT, EXACT><<<grid, 64 * NW, lds, s>>>(a);

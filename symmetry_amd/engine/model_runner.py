@@ -538,6 +538,9 @@ class ModelRunner:
         self._fill(lay, hn, [], [])
         dev.copy_(host[:lay.size])
         fb = self._forward_batch(kind, lay, dev, lay.nseq, filtered=filtered, need_logits=need_logits, sample=sample)
+        # a bucket captured in the middle of pipelined decode (its first use): the warmup runs sample into last_ids,
+        # which still holds the in-flight step's samples that the next replay's rows read as their input tokens
+        saved_ids = self.model.last_ids.clone()
         # eager warmup: allocates workspace and loads kernels outside the capture
         s = torch.cuda.Stream()
         s.wait_stream(torch.cuda.current_stream())
@@ -552,6 +555,7 @@ class ModelRunner:
         with torch.cuda.graph(g, pool=self._graph_pool):
             out = self.model.forward(fb, self.kv)
         torch.cuda.synchronize()
+        self.model.last_ids.copy_(saved_ids)
         exec_ = 0
         if _native.available() and os.environ.get("SYMMETRY_GRAPH_LAUNCH", "native") == "native":
             try:

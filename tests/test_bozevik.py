@@ -482,6 +482,35 @@ def test_greedy_generation_through_the_scheduler(tmp_path, device, dtype):
     assert eng.blocks.num_free == eng.blocks.num_blocks - 1 and eng.slots.num_free == 3
 
 
+@pytest.mark.parametrize("device", DEVICES)
+def test_preemption_and_abort_return_blocks_and_slots(tmp_path, device):
+    """A pool too small for every sequence's decoded tail: the scheduler preempts (blocks and state slot go back, the
+    sequence is recomputed from its first token later, its carried state rebuilt by that prefill) and the outputs
+    still follow the oracle; an aborted request frees its slot for a waiting one."""
+    device = _device(device)
+    cfg = _cfg_a()
+    path, tensors = _checkpoint(tmp_path, cfg, seed=13)
+    eng = _engine(path, device, "float32", blocks=8, seqs=3, max_num_batched_tokens=64)
+    prompts = [_tokens(n, cfg["vocab"], 40 + i) for i, n in enumerate((30, 25, 33, 12))]
+    seqs = [eng.add_request(f"p{i}", p, SamplingParams(max_tokens=28, ignore_eos=True)) for i, p in enumerate(prompts)]
+    steps = 0
+    while eng.has_unfinished() and steps < 3000:
+        eng.step()
+        steps += 1
+        if steps == 6:
+            eng.abort("p1")
+    assert sum(s.num_preemptions for s in seqs) > 0
+    for i, (p, s) in enumerate(zip(prompts, seqs)):
+        if i == 1:
+            continue
+        assert len(s.output_ids) == 28
+        lg = _oracle(cfg, tensors, p + s.output_ids[:-1])
+        for j, t in enumerate(s.output_ids):
+            row = lg[len(p) - 1 + j]
+            assert float(row.max() - row[t]) <= 1e-3 * float(row.std()), (i, j, t, int(row.argmax()))
+    assert eng.blocks.num_free == eng.blocks.num_blocks - 1 and eng.slots.num_free == 3
+
+
 def test_registered_config_and_checkpoint_roundtrip(tmp_path):
     from symmetry_amd.models.config import bozevik_from_config, bozevik_to_config, resolve
     from symmetry_amd.models.weights import random_weights, save_bozevik_checkpoint
