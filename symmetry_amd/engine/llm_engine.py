@@ -208,9 +208,13 @@ class LLMEngine:
                 import json
 
                 from ..models.config import from_config_json
+                from ..models.weights import safetensors_shapes
 
                 with open(path) as f:
-                    return from_config_json(json.load(f), name=cfg.model)
+                    conf = json.load(f)
+                # (designs that leave some sizes to the tensors get the checkpoint's header; HF checkpoints may be sharded)
+                shapes = safetensors_shapes(cfg.weights) if conf.get("architecture") == "Lemunex" else None
+                return from_config_json(conf, name=cfg.model, shapes=shapes)
         return resolve(cfg.model)
 
     def _max_decode_rows(self, mcfg: ModelConfig) -> int:

@@ -7,6 +7,10 @@ def model_class(cfg):
         from .bozevik import BozevikLM
 
         return BozevikLM
+    if family == "lemunex":
+        from .lemunex import LemunexLM
+
+        return LemunexLM
     if family == "llama":
         from .transformer import TransformerLM
 

@@ -255,6 +255,285 @@ SMALL_BOZEVIK_MOE = _bozevik_stack("small-bozevik-moe", 32768, 2048, 4, heads=16
                                    kv_rank=512, q_rank=1536, ff=8192, experts=16, top=4, expert_ff=1024, shared_ff=2048,
                                    max_position=8192, bos_token_id=32000, eos_token_ids=(32001, 32002))
 
+# --------------------------------------------------------------------------------------------------
+# Lemunex: parallel layers (one norm feeds the mixer and the feed-forward, both added to the stream).  Mixers: windowed
+# softmax attention beside gated linear attention ("parallel"), or a state-space layer ("mamba2"); feed-forward:
+# squared-ReLU, or routed gated experts with identity experts and a gated shared expert.
+# --------------------------------------------------------------------------------------------------
+@dataclass(frozen=True)
+class RotarySpec:
+    """Interleaved-pair rotary on the first ``dims`` entries of a head.  ``factor`` > 0 with ``original`` / ``fast`` /
+    ``slow`` set: frequencies are blended towards f / factor between the pairs that turn ``fast`` and ``slow`` times
+    over ``original`` positions, and cos / sin are scaled by 0.1 ln(factor) + 1."""
+    dims: int
+    base: float
+    factor: float = 0.0          # 0: no frequency scaling
+    original: float = 0.0
+    fast: float = 0.0
+    slow: float = 0.0
+
+
+@dataclass(frozen=True)
+class WindowAttnSpec:
+    heads: int
+    kv_heads: int
+    dim: int
+    vdim: int
+    window: int                  # a position sees itself and the window - 1 positions before it
+    scale: float
+    rot: RotarySpec
+
+
+@dataclass(frozen=True)
+class GatedLinearAttnSpec:
+    heads: int
+    dim: int
+    vdim: int
+    tau: float                   # decay = sigmoid(z) ** (1 / tau)
+    decay_rank: int              # inner size of the low-rank decay projection (from the checkpoint's tensor shapes)
+
+
+@dataclass(frozen=True)
+class PairMixerSpec:
+    """Two mixers side by side on the same input: scale_left * attention + scale_right * linear attention."""
+    left: WindowAttnSpec
+    right: GatedLinearAttnSpec
+    left_scale: float
+    right_scale: float
+
+
+@dataclass(frozen=True)
+class StateSpaceSpec:
+    heads: int
+    vdim: int
+    state: int
+    groups: int
+    conv: int                    # taps of the causal convolution
+    norm_groups: int
+
+    @property
+    def inner(self) -> int:
+        return self.heads * self.vdim
+
+    @property
+    def conv_channels(self) -> int:
+        return self.inner + 2 * self.groups * self.state
+
+
+@dataclass(frozen=True)
+class ReluSqSpec:
+    ff: int
+
+
+@dataclass(frozen=True)
+class RoutedSpec:
+    """Softmax router over experts + identity experts; choice by score + correction, weights = the plain scores."""
+    experts: int                 # experts that have tensors
+    identity: int                # further router outputs whose "expert" returns its input
+    top: int
+    expert_ff: int
+    shared_ff: int = 0           # 0: no shared expert
+
+
+@dataclass(frozen=True)
+class LemunexLayer:
+    type: str                    # "parallel" | "mamba2"
+    mixer: PairMixerSpec | StateSpaceSpec
+    mlp: ReluSqSpec | RoutedSpec | None = None
+
+
+@dataclass(frozen=True)
+class LemunexConfig:
+    family = "lemunex"
+    name: str
+    vocab_size: int
+    hidden_size: int
+    layers: tuple
+    norm_eps: float = 1e-5
+    max_position: int = 131072
+    bos_token_id: int = 1
+    eos_token_ids: tuple = (2,)
+    chat_format: str = "llama3"
+    tie_embeddings = False
+    rope_scaling = None
+
+    @property
+    def num_layers(self) -> int:
+        return len(self.layers)
+
+    @property
+    def is_moe(self) -> bool:
+        return any(isinstance(layer.mlp, RoutedSpec) for layer in self.layers)
+
+    def attn_layers(self) -> list:
+        """Layers that own planes of the paged key / value cache, in order."""
+        return [i for i, layer in enumerate(self.layers) if layer.type == "parallel"]
+
+    def num_params(self) -> int:
+        from .weights import lemunex_shapes
+
+        n = 0
+        for shape in lemunex_shapes(self).values():
+            k = 1
+            for v in shape:
+                k *= v
+            n += k
+        return n
+
+    def kv_bytes_per_token(self, dtype_bytes: int = 2) -> int:
+        return sum(self.layers[i].mixer.left.kv_heads * (self.layers[i].mixer.left.dim + self.layers[i].mixer.left.vdim)
+                   for i in self.attn_layers()) * dtype_bytes
+
+    def state_bytes_per_seq(self, dtype_bytes: int = 2) -> int:
+        n = 0
+        for layer in self.layers:
+            m = layer.mixer
+            if layer.type == "parallel":
+                n += m.right.heads * m.right.dim * m.right.vdim * 4
+            else:
+                n += m.heads * m.state * m.vdim * 4 + (m.conv - 1) * m.conv_channels * dtype_bytes
+        return n
+
+    def replace(self, **kw) -> "LemunexConfig":
+        return dataclasses.replace(self, **kw)
+
+
+def _take(d: dict, where: str, *keys, optional=()):
+    """The values of ``keys`` (+ optional ones, None if absent); any other key in ``d`` is a mechanism this reader
+    does not know, so it raises."""
+    d = dict(d)
+    out = [d.pop(k) for k in keys] + [d.pop(k, None) for k in optional]
+    if d:
+        raise ValueError(f"{where}: unknown keys {sorted(d)}")
+    return out
+
+
+def lemunex_from_config(cfg: dict, name: str = "lemunex", shapes: dict | None = None) -> LemunexConfig:
+    """config.json of a Lemunex checkpoint.  ``shapes`` (tensor name -> shape, the checkpoint's header) supplies the
+    sizes the configuration leaves to the tensors (the rank of the decay projection)."""
+    layers = []
+    for i, L in enumerate(cfg["layers"]):
+        kind, mixer, mlp = _take(L, f"layer {i}", "type", "mixer", optional=("mlp",))
+        if kind == "parallel":
+            left, right, ls, rs = _take(mixer, f"layer {i} mixer", "left", "right", "left_scale", "right_scale")
+            dim, heads, kvh, mask, rot, scale, vdim = _take(left, f"layer {i} left", "dim", "heads", "kv_heads", "mask",
+                                                            "rot", "scale", "vdim")
+            (window,) = _take(mask, f"layer {i} mask", "size")
+            base, dims, scaling = _take(rot, f"layer {i} rot", "base", "dims", optional=("scaling",))
+            if scaling:
+                factor, fast, orig, slow = _take(scaling, f"layer {i} rot.scaling", "factor", "fast", "original", "slow")
+                rspec = RotarySpec(int(dims), float(base), float(factor), float(orig), float(fast), float(slow))
+            else:
+                rspec = RotarySpec(int(dims), float(base))
+            lspec = WindowAttnSpec(int(heads), int(kvh), int(dim), int(vdim), int(window), float(scale), rspec)
+            if lspec.heads % lspec.kv_heads or rspec.dims % 2 or rspec.dims > lspec.dim or lspec.window < 1:
+                raise ValueError(f"layer {i}: heads {heads} / kv_heads {kvh} / rot.dims {dims} / dim {dim} do not fit")
+            rdim, rheads, tau, rvdim = _take(right, f"layer {i} right", "dim", "heads", "tau", "vdim")
+            key = f"l{i}.mix.right.a1"
+            if shapes is None or key not in shapes:
+                raise ValueError(f"layer {i}: the decay projection's rank comes from the shape of {key}")
+            rspec2 = GatedLinearAttnSpec(int(rheads), int(rdim), int(rvdim), float(tau), int(shapes[key][0]))
+            mix = PairMixerSpec(lspec, rspec2, float(ls), float(rs))
+        elif kind == "mamba2":
+            conv, groups, heads, ng, state, vdim = _take(mixer, f"layer {i} mixer", "conv", "groups", "heads",
+                                                         "norm_groups", "state", "vdim")
+            mix = StateSpaceSpec(int(heads), int(vdim), int(state), int(groups), int(conv), int(ng))
+            if mix.heads % mix.groups or mix.inner % mix.norm_groups or mix.conv < 1:
+                raise ValueError(f"layer {i}: heads {heads} / groups {groups} / norm_groups {ng} do not fit")
+        else:
+            raise ValueError(f"layer {i}: unknown layer type {kind!r}")
+        if mlp is None:
+            ff = None
+        elif mlp.get("kind") == "dense":
+            (_, f) = _take(mlp, f"layer {i} mlp", "kind", "ff")
+            ff = ReluSqSpec(int(f))
+        elif mlp.get("kind") == "moe":
+            _, expert, router, shared = _take(mlp, f"layer {i} mlp", "kind", "expert", "router", optional=("shared",))
+            (eff,) = _take(expert, f"layer {i} mlp.expert", "ff")
+            experts, top, ident = _take(router, f"layer {i} mlp.router", "experts", "top", optional=("identity",))
+            sff = _take(shared, f"layer {i} mlp.shared", "ff")[0] if shared else 0
+            ff = RoutedSpec(int(experts), int(ident or 0), int(top), int(eff), int(sff))
+            if not 1 <= ff.top <= ff.experts + ff.identity:
+                raise ValueError(f"layer {i}: top {top} of {ff.experts + ff.identity} router outputs")
+        else:
+            raise ValueError(f"layer {i}: unknown mlp kind {mlp.get('kind')!r}")
+        layers.append(LemunexLayer(kind, mix, ff))
+    vocab, width, norm, _, _, bos, eos = _take(cfg, "config", "vocab", "width", "norm", "layers",
+                                               optional=("architecture", "bos_token_id", "eos_token_ids"))
+    (eps,) = _take(norm, "norm", "eps")
+    return LemunexConfig(name=name, vocab_size=int(vocab), hidden_size=int(width), layers=tuple(layers),
+                         norm_eps=float(eps), bos_token_id=int(bos if bos is not None else 1),
+                         eos_token_ids=tuple(eos) if eos is not None else (2,))
+
+
+def lemunex_to_config(c: LemunexConfig) -> dict:
+    """The config.json form of a LemunexConfig (exports, tests)."""
+    layers = []
+    for layer in c.layers:
+        m = layer.mixer
+        if layer.type == "parallel":
+            a, g = m.left, m.right
+            rot = {"base": a.rot.base, "dims": a.rot.dims}
+            if a.rot.factor > 0:
+                rot["scaling"] = {"factor": a.rot.factor, "fast": a.rot.fast, "original": a.rot.original,
+                                  "slow": a.rot.slow}
+            md = {"left": {"dim": a.dim, "heads": a.heads, "kv_heads": a.kv_heads, "mask": {"size": a.window},
+                           "rot": rot, "scale": a.scale, "vdim": a.vdim},
+                  "left_scale": m.left_scale,
+                  "right": {"dim": g.dim, "heads": g.heads, "tau": g.tau, "vdim": g.vdim},
+                  "right_scale": m.right_scale}
+        else:
+            md = {"conv": m.conv, "groups": m.groups, "heads": m.heads, "norm_groups": m.norm_groups, "state": m.state,
+                  "vdim": m.vdim}
+        f = layer.mlp
+        if f is None:
+            fd = None
+        elif isinstance(f, ReluSqSpec):
+            fd = {"ff": f.ff, "kind": "dense"}
+        else:
+            fd = {"expert": {"ff": f.expert_ff}, "kind": "moe",
+                  "router": {"experts": f.experts, "identity": f.identity, "top": f.top}}
+            if f.shared_ff:
+                fd["shared"] = {"ff": f.shared_ff}
+        layers.append({"mixer": md, "mlp": fd, "type": layer.type})
+    return {"architecture": "Lemunex", "layers": layers, "norm": {"eps": c.norm_eps}, "vocab": c.vocab_size,
+            "width": c.hidden_size}
+
+
+def lemunex_stack(name, vocab, width, pattern, heads, kv_heads, dim, window, gla_heads, gla_dim, gla_vdim, ssm_heads,
+                  ssm_vdim, ssm_state, ff, experts=0, top=2, identity=0, expert_ff=0, shared_ff=0, decay_rank=16,
+                  ssm_groups=1, **kw) -> LemunexConfig:
+    """A stack from a pattern string: "P" parallel layer (attention + linear attention), "M" state-space layer;
+    lower case = that layer with the dense feed-forward, upper case with the routed one (if ``experts`` > 0)."""
+    layers = []
+    for ch in pattern:
+        if ch in "Pp":
+            rot = RotarySpec(dim // 2, 10000.0, 4.0, 4096.0, 32.0, 1.0)
+            mix = PairMixerSpec(WindowAttnSpec(heads, kv_heads, dim, dim, window, dim ** -0.5, rot),
+                                GatedLinearAttnSpec(gla_heads, gla_dim, gla_vdim, 16.0, decay_rank), 0.5, 0.5)
+            kind = "parallel"
+        else:
+            mix = StateSpaceSpec(ssm_heads, ssm_vdim, ssm_state, ssm_groups, 4, 1)
+            kind = "mamba2"
+        routed = experts > 0 and ch.isupper()
+        mlp = RoutedSpec(experts, identity, top, expert_ff, shared_ff) if routed else ReluSqSpec(ff)
+        layers.append(LemunexLayer(kind, mix, mlp))
+    return LemunexConfig(name=name, vocab_size=vocab, hidden_size=width, layers=tuple(layers), **kw)
+
+
+TINY_LEMUNEX = lemunex_stack("tiny-lemunex", 512, 128, "pMMP", heads=4, kv_heads=2, dim=32, window=48, gla_heads=2,
+                             gla_dim=16, gla_vdim=32, ssm_heads=4, ssm_vdim=16, ssm_state=16, ff=256, experts=6, top=2,
+                             identity=1, expert_ff=64, shared_ff=64, decay_rank=8, max_position=2048, bos_token_id=500,
+                             eos_token_ids=(501, 502))
+# layer shapes of a mid-size hybrid model (benchmarks; random weights)
+SMALL_LEMUNEX = lemunex_stack("small-lemunex", 32768, 2048, "pmmp", heads=16, kv_heads=4, dim=128, window=1024,
+                              gla_heads=8, gla_dim=128, gla_vdim=256, ssm_heads=64, ssm_vdim=64, ssm_state=128, ff=8192,
+                              max_position=8192, bos_token_id=32000, eos_token_ids=(32001, 32002))
+SMALL_LEMUNEX_MOE = lemunex_stack("small-lemunex-moe", 32768, 2048, "PMMP", heads=16, kv_heads=4, dim=128, window=1024,
+                                  gla_heads=8, gla_dim=128, gla_vdim=256, ssm_heads=64, ssm_vdim=64, ssm_state=128,
+                                  ff=8192, experts=16, top=4, identity=2, expert_ff=1024, shared_ff=2048,
+                                  max_position=8192, bos_token_id=32000, eos_token_ids=(32001, 32002))
+
 LLAMA31_SCALING = {
     "rope_type": "llama3",
     "factor": 8.0,
@@ -296,7 +575,8 @@ SMALL_LLAMA = ModelConfig(
 _REGISTRY = {
     c.name: c
     for c in (LLAMA3_8B, LLAMA31_8B, LLAMA3_70B, LLAMA31_70B, MIXTRAL_8X7B, TINY_LLAMA, TINY_MIXTRAL, SMALL_LLAMA,
-              TINY_LLAMA_KV8, TINY_MIXTRAL_E8, TINY_BOZEVIK, SMALL_BOZEVIK, SMALL_BOZEVIK_MOE)
+              TINY_LLAMA_KV8, TINY_MIXTRAL_E8, TINY_BOZEVIK, SMALL_BOZEVIK, SMALL_BOZEVIK_MOE, TINY_LEMUNEX,
+              SMALL_LEMUNEX, SMALL_LEMUNEX_MOE)
 }
 _ALIASES = {
     "llama3": "llama3:8b",
@@ -327,11 +607,14 @@ def known_models() -> list[str]:
     return sorted(set(_REGISTRY) | set(_ALIASES))
 
 
-def from_config_json(cfg: dict, name: str = "hf"):
+def from_config_json(cfg: dict, name: str = "hf", shapes: dict | None = None):
     """The model configuration of a checkpoint directory's config.json: the design is chosen by its
-    ``architecture`` key (Bozevik), otherwise the HuggingFace Llama / Mixtral keys."""
+    ``architecture`` key (Bozevik, Lemunex), otherwise the HuggingFace Llama / Mixtral keys.  ``shapes``: the
+    checkpoint's tensor shapes, for designs that leave some sizes to them."""
     if cfg.get("architecture") == "Bozevik":
         return bozevik_from_config(cfg, name)
+    if cfg.get("architecture") == "Lemunex":
+        return lemunex_from_config(cfg, name, shapes)
     return from_hf_config(cfg, name)
 
 

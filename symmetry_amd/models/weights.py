@@ -180,6 +180,8 @@ def random_weights(cfg: ModelConfig, shard: ShardSpec | None = None, device="cpu
     shard = shard or ShardSpec()
     if getattr(cfg, "family", "llama") == "bozevik":
         return bozevik_random_weights(cfg, shard, device, dtype, seed)
+    if getattr(cfg, "family", "llama") == "lemunex":
+        return lemunex_random_weights(cfg, shard, device, dtype, seed)
     shard.validate(cfg)
     shapes = full_shapes(cfg)
     tensors = {}
@@ -234,6 +236,8 @@ def load_hf_weights(path: str, cfg: ModelConfig, shard: ShardSpec | None = None,
     shard = shard or ShardSpec()
     if getattr(cfg, "family", "llama") == "bozevik":
         return load_bozevik_weights(path, cfg, shard, device, dtype)
+    if getattr(cfg, "family", "llama") == "lemunex":
+        return load_lemunex_weights(path, cfg, shard, device, dtype)
     shard.validate(cfg)
     wmap = _hf_index(path)
     handles = {}
@@ -396,5 +400,138 @@ def save_bozevik_checkpoint(weights: ModelWeights, path: str) -> None:
     os.makedirs(path, exist_ok=True)
     with open(os.path.join(path, "config.json"), "w") as f:
         json.dump(bozevik_to_config(weights.cfg), f, indent=1)
+    save_file({k: v.detach().to(torch.bfloat16).contiguous().cpu() for k, v in weights.tensors.items()},
+              os.path.join(path, "model.safetensors"))
+
+
+# --------------------------------------------------------------------------------------------------
+# Lemunex checkpoints: tensors keep the checkpoint's names (embed, embed.norm, l<i>.norm1, l<i>.mix.left.q,
+# l<i>.mix.in, l<i>.mlp.e<j>.gate, ..., final.norm, head); models/lemunex.py fuses what its GEMMs read.
+# --------------------------------------------------------------------------------------------------
+def safetensors_shapes(path: str) -> dict:
+    """Tensor name -> shape from the header of ``path``/model.safetensors (8-byte little-endian length + JSON)."""
+    import struct
+
+    with open(os.path.join(path, "model.safetensors"), "rb") as f:
+        (n,) = struct.unpack("<Q", f.read(8))
+        head = json.loads(f.read(n))
+    return {k: tuple(v["shape"]) for k, v in head.items() if k != "__metadata__"}
+
+
+def lemunex_shapes(cfg) -> dict:
+    from .config import ReluSqSpec, RoutedSpec
+
+    d = cfg.hidden_size
+    shapes = {"embed": (cfg.vocab_size, d), "embed.norm": (d,), "final.norm": (d,), "head": (cfg.vocab_size, d)}
+    for i, layer in enumerate(cfg.layers):
+        p, m = f"l{i}.", layer.mixer
+        shapes[p + "norm1"] = (d,)
+        if layer.type == "parallel":
+            a, g, q = m.left, m.right, p + "mix."
+            for nm, rows in (("q", a.heads * a.dim), ("k", a.kv_heads * a.dim), ("v", a.kv_heads * a.vdim)):
+                shapes[f"{q}left.{nm}"], shapes[f"{q}left.{nm}.b"] = (rows, d), (rows,)
+            shapes[q + "left.g"] = (a.heads, d)
+            shapes[q + "left.o"], shapes[q + "left.o.b"] = (d, a.heads * a.vdim), (d,)
+            shapes[q + "right.q"] = shapes[q + "right.k"] = (g.heads * g.dim, d)
+            shapes[q + "right.v"] = shapes[q + "right.g"] = (g.heads * g.vdim, d)
+            shapes[q + "right.o"] = (d, g.heads * g.vdim)
+            shapes[q + "right.norm"] = (g.vdim,)
+            shapes[q + "right.a1"] = (g.decay_rank, d)
+            shapes[q + "right.a2"], shapes[q + "right.a2.b"] = (g.heads * g.dim, g.decay_rank), (g.heads * g.dim,)
+        else:
+            q = p + "mix."
+            shapes[q + "in"] = (2 * m.inner + 2 * m.groups * m.state + m.heads, d)
+            shapes[q + "conv"], shapes[q + "conv.b"] = (m.conv_channels, m.conv), (m.conv_channels,)
+            shapes[q + "dt_bias"] = shapes[q + "A_log"] = shapes[q + "D"] = (m.heads,)
+            shapes[q + "norm"] = (m.inner,)
+            shapes[q + "o"] = (d, m.inner)
+
+        def glu(prefix, f):
+            shapes[prefix + "gate"], shapes[prefix + "up"], shapes[prefix + "down"] = (f, d), (f, d), (d, f)
+
+        f = layer.mlp
+        if isinstance(f, ReluSqSpec):
+            shapes[p + "mlp.up"], shapes[p + "mlp.down"] = (f.ff, d), (d, f.ff)
+        elif isinstance(f, RoutedSpec):
+            for e in range(f.experts):
+                glu(f"{p}mlp.e{e}.", f.expert_ff)
+            shapes[p + "mlp.router"] = (f.experts + f.identity, d)
+            shapes[p + "mlp.correction"] = (f.experts + f.identity,)
+            if f.shared_ff:
+                glu(p + "mlp.shared.", f.shared_ff)
+                shapes[p + "mlp.shared.sg"] = (1, d)
+    return shapes
+
+
+def lemunex_random_weights(cfg, shard: ShardSpec | None = None, device="cpu", dtype=torch.bfloat16,
+                           seed: int = 0) -> ModelWeights:
+    """Random init (benchmarks, tests): matrices N(0, (1.28 / sqrt(fan_in))^2); norm offsets, biases and router
+    corrections small and nonzero (so a dropped one shows); decay / step-size parameters in the ranges where the
+    recurrences remember hundreds of tokens."""
+    shard = shard or ShardSpec()
+    if shard.tp_size > 1 or shard.ep_size > 1:
+        raise NotImplementedError("Lemunex runs on one GPU per replica (its tensors are not sharded)")
+    tensors = {}
+    for name, shape in lemunex_shapes(cfg).items():
+        g = torch.Generator().manual_seed(_seed(seed, name))
+        leaf = name.rsplit(".", 1)[-1]
+        if name.endswith("right.norm") or name.endswith("mix.norm"):
+            t = 1.0 + 0.1 * torch.randn(shape, generator=g)
+        elif leaf in ("norm", "norm1"):
+            t = 0.1 * torch.randn(shape, generator=g)
+        elif name.endswith("a2.b"):
+            t = 3.0 + torch.randn(shape, generator=g)            # sigmoid(z) near one: slow decay
+        elif leaf == "b":
+            t = 0.1 * torch.randn(shape, generator=g)
+        elif leaf == "correction":
+            t = 0.02 * torch.randn(shape, generator=g)
+        elif leaf == "dt_bias":
+            t = -2.0 + torch.rand(shape, generator=g)
+        elif leaf == "A_log":
+            t = torch.log(0.05 + 0.5 * torch.rand(shape, generator=g))
+        elif leaf == "D":
+            t = 0.5 + torch.rand(shape, generator=g)
+        elif leaf == "conv":
+            t = torch.randn(shape, generator=g) * shape[1] ** -0.5
+        else:
+            tensors[name] = _randn(shape, _seed(seed, name), device, dtype, 1.0 if name == "embed" else _std(name, shape))
+            continue
+        tensors[name] = t.to(dtype).to(device)
+    return ModelWeights(cfg, shard, tensors)
+
+
+def load_lemunex_weights(path: str, cfg, shard: ShardSpec | None = None, device="cpu",
+                         dtype=torch.bfloat16) -> ModelWeights:
+    """model.safetensors of a Lemunex checkpoint directory; every tensor the configuration implies must be there
+    with the implied shape, and no other.  Tensors stay in the file's precision (the model converts what it fuses)."""
+    from safetensors import safe_open
+
+    shard = shard or ShardSpec()
+    if shard.tp_size > 1 or shard.ep_size > 1:
+        raise NotImplementedError("Lemunex runs on one GPU per replica (its tensors are not sharded)")
+    shapes = lemunex_shapes(cfg)
+    tensors = {}
+    with safe_open(os.path.join(path, "model.safetensors"), framework="pt") as f:
+        names = set(f.keys())
+        missing, extra = sorted(set(shapes) - names), sorted(names - set(shapes))
+        if missing or extra:
+            raise ValueError(f"checkpoint does not fit its config: missing {missing[:4]}, unexpected {extra[:4]}")
+        for name, shape in shapes.items():
+            t = f.get_tensor(name)
+            if tuple(t.shape) != tuple(shape):
+                raise ValueError(f"{name}: shape {tuple(t.shape)}, the config implies {tuple(shape)}")
+            tensors[name] = t.to(device)
+    return ModelWeights(cfg, shard, tensors)
+
+
+def save_lemunex_checkpoint(weights: ModelWeights, path: str) -> None:
+    """config.json + model.safetensors (bf16) of a Lemunex model, in the form the loader reads."""
+    from safetensors.torch import save_file
+
+    from .config import lemunex_to_config
+
+    os.makedirs(path, exist_ok=True)
+    with open(os.path.join(path, "config.json"), "w") as f:
+        json.dump(lemunex_to_config(weights.cfg), f, indent=1)
     save_file({k: v.detach().to(torch.bfloat16).contiguous().cpu() for k, v in weights.tensors.items()},
               os.path.join(path, "model.safetensors"))

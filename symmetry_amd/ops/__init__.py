@@ -705,3 +705,153 @@ def gather_sum(y, dst, k, extra, out):
     if _gpu(out):
         return _lat().gather_sum(y, dst, int(k), extra, out)
     return reference.gather_sum(y, dst, k, extra, out)
+
+
+# ======================================================================================================
+# Mechanisms of the hybrid model family (csrc/kernels/hybrid_rows.hip, window_attention.hip, decay_scan.hip):
+# windowed softmax attention with grouped key / value heads over a paged cache, linear recurrences with decaying
+# state (per key channel or per head), causal convolutions with carried taps, parallel feed-forward, a softmax
+# router with identity experts.  Inputs that are column ranges of one fused projection are passed as views (unit
+# inner stride); activations bf16 or fp32, the stream / states / statistics / scores / decays fp32.
+# ======================================================================================================
+def _hyb():
+    return _native.hybrid_ops()
+
+
+def embed_norm(ids, table, w, eps, offset, x, src=None, prev=None):
+    """x (fp32) = table[token] / rms * (offset + w); rows with src >= 0 take the token prev[src]."""
+    if _gpu(x):
+        return _hyb().embed_norm(ids, src, prev, table, w, float(eps), float(offset), x)
+    return reference.embed_norm(reference.resolve_ids(ids, src, prev), table, w, eps, offset, x)
+
+
+def rms_norm_rows(x, rows, w, eps, offset, out):
+    """out[i] = x[rows[i]] / rms * (offset + w) (rows None: the first len(out) rows); x fp32."""
+    if _gpu(x):
+        return _hyb().rms_norm_rows(x, rows, w, float(eps), float(offset), out)
+    return reference.rms_norm_rows(x, rows, w, eps, offset, out)
+
+
+def residual_mix_norm(x, a, sa, bias_a, b, sb, c, sc, w=None, eps=0.0, offset=0.0, out=None):
+    """x += sa * (a + bias_a) + sb * b + sc * c in fp32 (bias_a, b, c optional); with ``out``: out = x / rms * (offset
+    + w), the next layer's normalised input, from the same pass."""
+    if _gpu(x):
+        return _hyb().residual_mix_norm(x, a, float(sa), bias_a, b, float(sb), c, float(sc), w, float(eps),
+                                        float(offset), out)
+    return reference.residual_mix_norm(x, a, sa, bias_a, b, sb, c, sc, w, eps, offset, out)
+
+
+def rope_scaled_table(max_pos, dims, base, factor=0.0, original=0.0, fast=0.0, slow=0.0, device=None):
+    return reference.rope_scaled_table(max_pos, dims, base, factor, original, fast, slow, device)
+
+
+def qkv_rope_cache(z, bias, H, G, dk, dv, positions, slots, rope, q_out, k_cache, v_cache):
+    """z [T, H dk | G dk | G dv (| ...)] + bias (fp32) -> q_out [T, H, dk] and the token's rows of the paged caches
+    k [NB, BS, G, dk], v [NB, BS, G, dv] (slot >= 0); q and k turn by ``rope`` [max_pos, pairs, 2] on their first
+    2 * pairs entries (interleaved pairs), in fp32."""
+    if _gpu(z):
+        return _hyb().qkv_rope_cache(z, bias, int(H), int(G), int(dk), int(dv), positions, slots, rope, q_out,
+                                     k_cache, v_cache)
+    return reference.qkv_rope_cache(z, bias, H, G, dk, dv, positions, slots, rope, q_out, k_cache, v_cache)
+
+
+WINDOW_ATTN_IMPL = os.environ.get("SYMMETRY_WINDOW_ATTN", "auto")
+
+
+def window_attn(q, k_cache, v_cache, block_tables, row_seq, positions, window, scale, gate, out, tiles=None, cu_q=None):
+    """Softmax attention of q [T, H, dk] over the paged caches: row r sees positions max(0, p - window + 1) .. p of
+    sequence row_seq[r] (p = positions[r]); query head h reads key / value head h // (H / G); scores and weights
+    fp32.  ``gate`` [T, H] (a view): head outputs are multiplied by sigmoid(gate).  ``tiles`` / ``cu_q``: the packed
+    prompt form (64-row query tiles), for the tiled kernel."""
+    if _gpu(q):
+        return _hyb().window_attn(q, k_cache, v_cache, block_tables, row_seq, positions, int(window), float(scale), gate,
+                                  out, tiles, cu_q)
+    return reference.window_attn(q, k_cache, v_cache, block_tables, row_seq, positions, window, scale, gate, out)
+
+
+DECAY_CHANNEL_GATE, DECAY_STEP_SIZE = 0, 1
+
+
+def decay_scan(mode, q, k, v, dz, dbias, dparam, skip, q_scale, H, N, P, hpg, state, cu_q, prev_row, save_slot, runs,
+               out):
+    """Linear recurrence with decaying state, per head h over every run of rows (cu_q[i] .. cu_q[i + 1]; cu_q None:
+    every row its own run): S <- diag(a_t) S + b_t k_t v_t^T (S [N, P] fp32), out_t = S^T (q_scale q_t) (+ skip_h v_t).
+    DECAY_CHANNEL_GATE: a = sigmoid(dz + dbias) ** (1 / dparam) per key channel (dz [T, H N], dparam a number), b = 1;
+    DECAY_STEP_SIZE: b = softplus(dz + dbias[h]), a = exp(-exp(dparam[h]) b) per head (dz [T, H]).
+    q / k [T, (H / hpg) N]: head h reads group h // hpg.  A run starts from state[slot] if prev_row[first] <= -2
+    (slot = -(v + 2)), else from zero; it ends in state[save_slot[last]] (>= 0).  out fp32 [T, H, P]."""
+    if _gpu(out):
+        dp = dparam if torch.is_tensor(dparam) else None
+        return _hyb().decay_scan(int(mode), q, k, v, dz, dbias, dp, 0.0 if dp is not None else float(dparam), skip,
+                                 float(q_scale), int(H), int(N), int(P), int(hpg), state, cu_q, prev_row, save_slot,
+                                 int(runs), out)
+    return reference.decay_scan(mode, q, k, v, dz, dbias, dparam, skip, q_scale, H, N, P, hpg, state, cu_q, prev_row,
+                                save_slot, runs, out)
+
+
+def gated_group_norm(y, gate, w, eps, group, gate_first, out):
+    """y fp32 [T, C], gate [T, C] (view): s = silu(gate); gate_first: out = rms_group(y s) w, else rms_group(y) w s;
+    rms over groups of ``group`` columns; w [len] repeats over the columns (C % len == 0)."""
+    if _gpu(y):
+        return _hyb().gated_group_norm(y, gate, w, float(eps), int(group), bool(gate_first), out)
+    return reference.gated_group_norm(y, gate, w, eps, group, gate_first, out)
+
+
+def causal_conv_silu(xin, w, b, state, cu_q, prev_row, runs, out):
+    """out_t = silu(b + sum_j w[:, taps - 1 - j] x_(t - j)) per channel over every run; inputs before the run come from
+    state[slot] [taps - 1, C] (prev_row[first] <= -2) or are zero.  xin [T, C] (view)."""
+    if _gpu(out):
+        return _hyb().causal_conv_silu(xin, w, b, state, cu_q, prev_row, int(runs), out)
+    return reference.causal_conv_silu(xin, w, b, state, cu_q, prev_row, runs, out)
+
+
+def conv_state_update(xin, state, cu_q, prev_row, save_slot, runs):
+    """state[save_slot[last]] = the newest taps - 1 inputs of every run's sequence (older ones from its old state)."""
+    if _gpu(xin):
+        return _hyb().conv_state_update(xin, state, cu_q, prev_row, save_slot, int(runs))
+    return reference.conv_state_update(xin, state, cu_q, prev_row, save_slot, runs)
+
+
+def relu_sq(a, out):
+    if _gpu(out):
+        return _hyb().relu_sq(a, out)
+    return reference.relu_sq(a, out)
+
+
+def silu_mul(gate, up, out):
+    """out = silu(gate) * up; gate, up [R, F] views."""
+    if _gpu(out):
+        return _hyb().silu_mul(gate, up, out)
+    return reference.silu_mul(gate, up, out)
+
+
+def softmax_topk(x, Wr, corr, k, ids, w):
+    """Router: s = softmax(x @ Wr.T) in fp32 over all outputs; the k largest of s + corr -> ids [T, k]; w = their s."""
+    if _gpu(x):
+        return _hyb().softmax_topk(x, Wr, corr, int(k), ids, w)
+    return reference.softmax_topk(x, Wr, corr, k, ids, w)
+
+
+def moe_mix(y, dst, ids, w, k, E, h, shared, sgate, out):
+    """out[t] (fp32) = sum_j w[a] * (ids[a] >= E ? h[t] : y[dst[a]]), a = t k + j, + sigmoid(sgate[t]) * shared[t]."""
+    if _gpu(out):
+        return _hyb().moe_mix(y, dst, ids, w, int(k), int(E), h, shared, sgate, out)
+    return reference.moe_mix(y, dst, ids, w, k, E, h, shared, sgate, out)
+
+
+def hyb_expert_offsets(ids, R, E, offsets, cursor):
+    if _gpu(ids):
+        return _hyb().expert_offsets(ids, int(R), int(E), offsets, cursor)
+    return reference.expert_offsets(ids, R, E, offsets, cursor)
+
+
+def hyb_scatter_scaled(x, ids, w, k, offsets, cursor, xs, dst):
+    if _gpu(x):
+        return _hyb().scatter_scaled(x, ids, w, int(k), offsets, cursor, xs, dst)
+    return reference.scatter_scaled(x, ids, w, k, offsets, cursor, xs, dst)
+
+
+def hyb_grouped_linear(xs, W, offsets, y):
+    if _gpu(xs):
+        return _hyb().grouped_linear(xs, W, offsets, y)
+    return reference.grouped_linear(xs, W, offsets, y)

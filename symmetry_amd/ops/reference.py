@@ -699,3 +699,204 @@ def gather_sum(y, dst, k, extra, out) -> None:
     if extra is not None:
         s = s + extra.float().view_as(s)
     out.copy_(s)
+
+
+# ======================================================================================================
+# torch references of the hybrid family's ops (windowed attention beside decaying linear recurrences, state-space
+# layers, parallel feed-forward; csrc/kernels/hybrid_*.hip).  Same contracts as the kernels: outputs in place,
+# activations in the tensors' own dtype, everything the recurrences and statistics touch in fp32.
+# ======================================================================================================
+def _unit_rms(v, eps):
+    return v / torch.sqrt((v * v).mean(-1, keepdim=True) + eps)
+
+
+def embed_norm(ids, table, w, eps, offset, x) -> None:
+    x.copy_(_unit_rms(table[ids.long()].float(), eps) * (offset + w.float()))
+
+
+def rms_norm_rows(x, rows, w, eps, offset, out) -> None:
+    n = out.shape[0]
+    v = x[rows[:n].long()] if rows is not None else x[:n]
+    out.copy_((_unit_rms(v.float(), eps) * (offset + w.float())).to(out.dtype))
+
+
+def residual_mix_norm(x, a, sa, bias_a, b, sb, c, sc, w, eps, offset, out) -> None:
+    s = a.float().view_as(x)
+    if bias_a is not None:
+        s = s + bias_a.float()
+    s = sa * s
+    if b is not None:
+        s = s + sb * b.float().view_as(x)
+    if c is not None:
+        s = s + sc * c.float().view_as(x)
+    x.add_(s)
+    if out is not None:
+        out.copy_((_unit_rms(x, eps) * (offset + w.float())).to(out.dtype))
+
+
+def rope_scaled_table(max_pos: int, dims: int, base: float, factor: float, original: float, fast: float, slow: float,
+                      device=None) -> torch.Tensor:
+    """[max_pos, dims / 2, 2] fp32 (cos, sin) * magnitude of the angles p * f_i; with factor > 0 the frequencies are
+    blended towards f_i / factor over the pairs between the ones turning ``fast`` and ``slow`` times in ``original``
+    positions, and the magnitude is 0.1 ln(factor) + 1.  Angles are fp32 products, cos / sin evaluated in double."""
+    import math
+
+    i = torch.arange(dims // 2, dtype=torch.float64)
+    f = torch.tensor(float(base), dtype=torch.float64) ** (-2.0 * i / dims)
+    mag = 1.0
+    if factor > 0:
+        def at(turns):
+            return dims * math.log(original / (2.0 * math.pi * turns)) / (2.0 * math.log(base))
+
+        lo, hi = max(math.floor(at(fast)), 0), min(math.ceil(at(slow)), dims - 1)
+        ramp = ((i - lo) / max(hi - lo, 0.001)).clamp(0.0, 1.0)
+        f = f / factor * ramp + f * (1.0 - ramp)
+        mag = 0.1 * math.log(factor) + 1.0
+    a = (torch.arange(max_pos, dtype=torch.float32)[:, None] * f.float()[None, :]).double()
+    return (torch.stack([torch.cos(a), torch.sin(a)], -1) * mag).float().to(device or "cpu")
+
+
+def qkv_rope_cache(z, bias, H, G, dk, dv, positions, slots, rope, q_out, k_cache, v_cache) -> None:
+    T = z.shape[0]
+    nq, nk, nv = H * dk, G * dk, G * dv
+    zf = z[:, :nq + nk + nv].float() + bias.float()[:nq + nk + nv]
+    cs = rope[positions[:T].long()][:, None]                  # [T, 1, rot / 2, 2]
+    rot = 2 * rope.shape[1]
+
+    def turn(v):
+        return torch.cat([_rot_pairs(v[..., :rot], cs), v[..., rot:]], -1)
+
+    q_out.copy_(turn(zf[:, :nq].view(T, H, dk)).to(q_out.dtype))
+    k = turn(zf[:, nq:nq + nk].view(T, G, dk)).to(k_cache.dtype)
+    v = zf[:, nq + nk:].view(T, G, dv).to(v_cache.dtype)
+    sl = slots[:T].long()
+    keep = sl >= 0
+    k_cache.view(-1, G, dk)[sl[keep]] = k[keep]
+    v_cache.view(-1, G, dv)[sl[keep]] = v[keep]
+
+
+def window_attn(q, k_cache, v_cache, block_tables, row_seq, positions, window, scale, gate, out) -> None:
+    T, H, dk = q.shape
+    BS, G = k_cache.shape[1], k_cache.shape[2]
+    rep = H // G
+    for r in range(T):
+        p = int(positions[r])
+        j0 = max(0, p - window + 1)
+        bt = block_tables[int(row_seq[r])].long()
+        idx = torch.arange(j0, p + 1)
+        K = k_cache[bt[idx // BS], idx % BS].float()            # [n, G, dk]
+        V = v_cache[bt[idx // BS], idx % BS].float()
+        qr = q[r].float().view(G, rep, dk)
+        s = torch.einsum("grd,ngd->grn", qr, K) * scale
+        o = torch.einsum("grn,ngv->grv", torch.softmax(s, -1), V).reshape(H, -1)
+        if gate is not None:
+            o = o * torch.sigmoid(gate[r].float())[:, None]
+        out[r] = o.to(out.dtype)
+
+
+def _runs(T, cu_q, runs):
+    if cu_q is None:
+        return [(r, r + 1) for r in range(runs)]
+    cu = cu_q.tolist()
+    return [(cu[i], cu[i + 1]) for i in range(runs)]
+
+
+def decay_scan(mode, q, k, v, dz, dbias, dparam, skip, q_scale, H, N, P, hpg, state, cu_q, prev_row, save_slot, runs,
+               out) -> None:
+    """S <- diag(a_t) S + b_t k_t v_t^T, o_t = S^T (q_scale q_t) (+ skip_h v_t) per head over every run of rows.
+    mode 0: a = sigmoid(dz + dbias) ** (1 / dparam) per key channel, b = 1;
+    mode 1: b = softplus(dz + dbias[h]), a = exp(-exp(dparam[h]) * b) per head.  q / k of head h: group h // hpg."""
+    T = q.shape[0]
+    qf = q.float().reshape(T, -1, N) * q_scale
+    kf, vf = k.float().reshape(T, -1, N), v.float().reshape(T, H, P)
+    if mode == 0:
+        ls = torch.nn.functional.logsigmoid(dz.float().reshape(T, H, N) + dbias.float().view(H, N))
+        a = torch.exp(ls / float(dparam))                              # [T, H, N]
+        b = torch.ones(T, H)
+    else:
+        b = torch.nn.functional.softplus(dz.float().reshape(T, H) + dbias.float(), beta=1.0, threshold=1e9)
+        a = torch.exp(-torch.exp(dparam.float()) * b)[:, :, None].expand(T, H, N)
+    grp = torch.arange(H) // hpg
+    o = out.view(T, H, P)
+    for s0, s1 in _runs(T, cu_q, runs):
+        if s1 <= s0:
+            continue
+        pr = int(prev_row[s0])
+        S = state[-(pr + 2)].clone() if pr <= -2 else torch.zeros(H, N, P)
+        for t in range(s0, s1):
+            S = a[t][:, :, None] * S + (b[t][:, None] * kf[t, grp])[:, :, None] * vf[t][:, None, :]
+            y = torch.einsum("hnp,hn->hp", S, qf[t, grp])
+            if skip is not None:
+                y = y + skip.float()[:, None] * vf[t]
+            o[t] = y
+        sv = int(save_slot[s1 - 1])
+        if sv >= 0:
+            state[sv] = S
+
+
+def gated_group_norm(y, gate, w, eps, group, gate_first, out) -> None:
+    T, C = y.shape
+    g = gate.float()
+    g = g * torch.sigmoid(g)
+    v = y * g if gate_first else y
+    v = _unit_rms(v.view(T, C // group, group), eps).reshape(T, C)
+    v = v * w.float().repeat(C // w.numel())
+    out.copy_((v if gate_first else v * g).to(out.dtype))
+
+
+def causal_conv_silu(xin, w, b, state, cu_q, prev_row, runs, out) -> None:
+    T, C = out.shape
+    taps = w.shape[1]
+    wf, xf = w.float(), xin.float()
+    for s0, s1 in _runs(T, cu_q, runs):
+        if s1 <= s0:
+            continue
+        pr = int(prev_row[s0])
+        hist = state[-(pr + 2)].float() if pr <= -2 else torch.zeros(taps - 1, C)
+        full = torch.cat([hist, xf[s0:s1]], 0)
+        y = b.float()[None, :].expand(s1 - s0, -1).clone()
+        for j in range(taps):
+            y = y + full[j:j + s1 - s0] * wf[:, j]
+        out[s0:s1] = (y * torch.sigmoid(y)).to(out.dtype)
+
+
+def conv_state_update(xin, state, cu_q, prev_row, save_slot, runs) -> None:
+    T = xin.shape[0]
+    keep = state.shape[1]
+    for s0, s1 in _runs(T, cu_q, runs):
+        if s1 <= s0:
+            continue
+        sv = int(save_slot[s1 - 1])
+        if sv < 0:
+            continue
+        pr = int(prev_row[s0])
+        hist = state[-(pr + 2)] if pr <= -2 else torch.zeros_like(state[0])
+        state[sv] = torch.cat([hist, xin[s0:s1].to(state.dtype)], 0)[-keep:] if keep else hist
+
+
+def relu_sq(a, out) -> None:
+    out.copy_((torch.relu(a.float()) ** 2).to(out.dtype))
+
+
+def silu_mul(gate, up, out) -> None:
+    g = gate.float()
+    out.copy_((g * torch.sigmoid(g) * up.float()).to(out.dtype))
+
+
+def softmax_topk(x, Wr, corr, k, ids, w) -> None:
+    T = x.shape[0]
+    s = torch.softmax(x.float() @ Wr.float().t(), -1)
+    pick = torch.argsort(s + corr.float(), dim=-1, descending=True, stable=True)[:, :k]
+    ids[: T * k].copy_(pick.reshape(-1).int())
+    w[: T * k].copy_(torch.gather(s, 1, pick).reshape(-1))
+
+
+def moe_mix(y, dst, ids, w, k, E, h, shared, sgate, out) -> None:
+    T = out.shape[0]
+    e = ids[: T * k].long().view(T, k)
+    rows = y.float()[dst[: T * k].long()].view(T, k, -1)
+    rows = torch.where((e >= E)[:, :, None], h.float()[:, None, :], rows)
+    s = (w[: T * k].view(T, k, 1) * rows).sum(1)
+    if shared is not None:
+        s = s + torch.sigmoid(sgate.float()).view(T, 1) * shared.float().view_as(s)
+    out.copy_(s)
