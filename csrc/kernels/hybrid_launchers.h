@@ -1,0 +1,123 @@
+// Host-side launch entry points of the kernels in hybrid_rows.hip, window_attention.hip and decay_scan.hip: the
+// mechanisms of models that put windowed softmax attention beside linear recurrences with decaying state, use
+// state-space layers with a carried convolution, and add mixer and feed-forward to the stream from one norm.
+//
+// Every launcher enqueues on the given stream, allocates nothing and never synchronises (hipGraph-capturable).
+// Activations are bf16 or fp32 (`f32` flag: the whole model in 32-bit); the residual stream, recurrent states,
+// norm statistics, rotary angles, decays, step sizes, router scores and attention scores / weights are always fp32.
+// Inputs that are column ranges of a wider matrix carry their row stride (`ld`, in elements).  Shape preconditions
+// are checked by the op layer (csrc/bindings/hybrid_ops.cpp) before any launch.
+#pragma once
+#include <hip/hip_runtime.h>
+
+// ---- hybrid_rows.hip -----------------------------------------------------------------------------------
+// x[row] = table[token] / rms * (offset + w), token = src[row] >= 0 ? prev[src[row]] : ids[row]
+void launch_embed_norm(const int* ids, const int* src, const int* prev, const void* table, const float* w, float eps,
+                       float offset, float* x, int T, int d, int f32, hipStream_t s);
+// out[i] = x[rows ? rows[i] : i] / rms * (offset + w)
+void launch_rms_norm_rows(const float* x, const long long* rows, const float* w, float eps, float offset, void* out,
+                          int n, int d, int f32, hipStream_t s);
+// x += sa * (a + bias_a) + sb * b + sc * c (bias_a, b, c optional; each of a, b, c bf16 or fp32: *_f32);
+// out (optional, activation dtype) = x_new / rms * (offset + w)
+struct ResidualMixArgs {
+  float* x;
+  const void* a; int a_f32; float sa; const float* bias_a;
+  const void* b; int b_f32; float sb;
+  const void* c; int c_f32; float sc;
+  const float* w; float eps, offset;
+  void* out;
+  int T, d;
+};
+void launch_residual_mix_norm(const ResidualMixArgs& a, int f32, hipStream_t s);
+// z[t] = q (H dk) | k (G dk) | v (G dv), + bias; q and k turn on their first 2 * pairs entries by rope[pos][pair];
+// q -> q_out [T][H][dk]; k, v -> cache rows `slot` (>= 0) of k_cache [rows][G][dk], v_cache [rows][G][dv]
+struct QkvRopeArgs {
+  const void* z; long long ldz;
+  const float* bias;
+  int H, G, dk, dv, pairs;
+  const int* positions;
+  const int* slots;
+  const float* rope;   // [max_pos][pairs][2] cos, sin (scaled)
+  void* q_out;
+  void* k_cache;
+  void* v_cache;
+};
+void launch_qkv_rope_cache(const QkvRopeArgs& a, int T, int f32, hipStream_t s);
+// s = silu(gate); gate_first: out = rms_g(y s) w, else out = rms_g(y) w s; rms over groups of `group` columns,
+// w [wlen] repeating over the columns
+void launch_gated_group_norm(const float* y, const void* gate, long long ldg, const float* w, int wlen, float eps,
+                             int group, int gate_first, void* out, int T, int C, int f32, hipStream_t s);
+// run i = rows cu_q[i] .. cu_q[i + 1] (cu_q null: row i alone); inputs before a run: state[slot] [taps - 1][C] where
+// prev_row[first] <= -2 (slot = -(v + 2)), else zero.  out = silu(b + sum_j w[c][taps - 1 - j] x[t - j][c])
+struct ConvArgs {
+  const void* xin; long long ldx;
+  const void* w;       // [C][taps] activation dtype
+  const float* b;      // [C]
+  void* state;         // [slots][taps - 1][C] activation dtype
+  long long state_stride;
+  const int* cu_q;
+  const int* row_seq;
+  const int* prev_row;
+  const int* save_slot;
+  void* out;           // [T][C]
+  int T, C, taps, runs;
+};
+void launch_causal_conv_silu(const ConvArgs& a, int f32, hipStream_t s);
+void launch_conv_state_update(const ConvArgs& a, int f32, hipStream_t s);
+// out = relu(a)^2
+void launch_relu_sq(const void* a, long long lda, void* out, int R, int F, int f32, hipStream_t s);
+// out = silu(gate) * up
+void launch_silu_mul(const void* gate, long long ldg, const void* up, long long ldu, void* out, int R, int F, int f32,
+                     hipStream_t s);
+// s = softmax(x . Wr[e]) over En outputs (fp32); the k largest of s + corr (ties: lowest index) -> ids, w = their s
+void launch_softmax_topk(const void* x, const void* Wr, const float* corr, int T, int d, int En, int k, int* ids,
+                         float* w, int f32, hipStream_t s);
+// out[t] = sum_j w[a] * (ids[a] >= E ? h[t] : y[dst[a]]) + sigmoid(sgate[t]) * shared[t], a = t k + j
+void launch_moe_mix(const void* y, const int* dst, const int* ids, const float* w, int k, int E, const void* h,
+                    const void* shared, const void* sgate, long long ldsg, float* out, int T, int d, int f32,
+                    hipStream_t s);
+
+// ---- window_attention.hip ------------------------------------------------------------------------------
+struct WindowAttnArgs {
+  const void* q;        // [T][H][dk]
+  const void* k_cache;  // [blocks][BS][G][dk]
+  const void* v_cache;  // [blocks][BS][G][dv]
+  const int* block_tables;  // [seqs][max_blocks]
+  const int* row_seq;   // [T]
+  const int* positions; // [T]: row sees positions max(0, p - window + 1) .. p
+  const void* gate;     // [T][H] (row stride ldg) or null: output times sigmoid(gate)
+  long long ldg;
+  void* out;            // [T][H][dv]
+  int T, H, G, dk, dv, BS, max_blocks, window;
+  float scale;
+  // packed prompt form for the tiled kernel: 64-row query tiles (sequence, first row within the run)
+  const int* tiles;
+  const int* cu_q;
+  int ntiles;
+};
+// Returns the implementation used: 0 = one wave per (row, head) (all shapes, both dtypes), 1 = tiled MFMA (bf16).
+int launch_window_attn(const WindowAttnArgs& a, int f32, int impl, hipStream_t s);
+
+// ---- decay_scan.hip ------------------------------------------------------------------------------------
+struct DecayScanArgs {
+  int mode;             // 0: decay per key channel = sigmoid(dz + dbias)^(1 / tau); 1: step size b = softplus(dz +
+                        // dbias[h]), decay per head = exp(-exp(rate[h]) b), input scaled by b
+  const void* q; long long ldq;   // [T][(H / hpg) N]
+  const void* k; long long ldk;
+  const void* v; long long ldv;   // [T][H P]
+  const void* dz; long long ldd;  // mode 0: [T][H N]; mode 1: [T][H]
+  const float* dbias;   // mode 0: [H N]; mode 1: [H]
+  const float* rate;    // mode 1: [H]
+  float tau;            // mode 0
+  const float* skip;    // [H] or null: out += skip[h] * v
+  float q_scale;
+  int H, N, P, hpg;
+  float* state;         // [slots][H][N][P]
+  long long state_stride;
+  const int* cu_q;      // runs (null: every row its own run)
+  const int* prev_row;
+  const int* save_slot;
+  int runs, T;
+  float* out;           // [T][H][P]
+};
+void launch_decay_scan(const DecayScanArgs& a, int f32, hipStream_t s);

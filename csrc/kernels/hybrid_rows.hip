@@ -1,0 +1,376 @@
+// Row kernels of the hybrid model family (windowed attention beside linear recurrences, state-space layers, one norm
+// feeding mixer and feed-forward):
+//
+//   embed_norm          x = table[token] / rms * (offset + w)               (fp32 stream)
+//   rms_norm_rows       norm of (gathered) stream rows into the activation dtype
+//   residual_mix_norm   x += sa (a + bias) + sb b + sc c in fp32, and the next layer's normalised input from the same pass
+//   qkv_rope_cache      bias + scaled interleaved-pair rotary of q / k, paged key / value cache write
+//   gated_group_norm    silu gate and RMS norm over column groups, in either order
+//   causal_conv_silu    per-channel causal convolution over a run of rows with carried taps, + silu
+//   conv_state_update   the newest taps - 1 inputs of every run into its sequence's state slot
+//   relu_sq, silu_mul   feed-forward activations on column ranges of a fused projection
+//   softmax_topk        router: fp32 softmax over all outputs, choice by score + correction, weights = plain scores
+//   moe_mix             weighted sum of the chosen experts' rows (identity experts: the input row) + gated shared expert
+//
+// One workgroup per row unless noted; columns strided over the threads (coalesced), any width.  All statistics,
+// rotations, gates and sums are fp32; only the stored activations take the activation dtype T (bf16 or float).
+#include "common.h"
+#include "hybrid_launchers.h"
+
+namespace {
+
+constexpr int NT = 256;
+
+SYM_DEV float ldf(const void* p, int f32, long long i) {
+  return f32 ? reinterpret_cast<const float*>(p)[i] : (float)reinterpret_cast<const bf16*>(p)[i];
+}
+
+SYM_DEV float sigmoidf(float v) { return 1.f / (1.f + expf(-v)); }
+SYM_DEV float silu_exact(float v) { return v / (1.f + expf(-v)); }
+
+template <typename T>
+__global__ __launch_bounds__(NT) void embed_norm_kernel(const int* __restrict__ ids, const int* __restrict__ src,
+                                                        const int* __restrict__ prev, const T* __restrict__ table,
+                                                        const float* __restrict__ w, float eps, float offset,
+                                                        float* __restrict__ x, int d) {
+  __shared__ float scratch[NT / 64];
+  const int row = blockIdx.x;
+  const int sr = src ? src[row] : -1;
+  const long long tok = sr >= 0 ? prev[sr] : ids[row];
+  const T* t = table + tok * d;
+  float sq = 0.f;
+  for (int c = threadIdx.x; c < d; c += NT) {
+    const float v = (float)t[c];
+    sq += v * v;
+  }
+  const float r = 1.f / sqrtf(block_sum<NT>(sq, scratch) / (float)d + eps);
+  for (int c = threadIdx.x; c < d; c += NT) x[(long long)row * d + c] = (float)t[c] * r * (offset + w[c]);
+}
+
+template <typename T>
+__global__ __launch_bounds__(NT) void rms_norm_rows_kernel(const float* __restrict__ x, const long long* __restrict__ rows,
+                                                           const float* __restrict__ w, float eps, float offset,
+                                                           T* __restrict__ out, int d) {
+  __shared__ float scratch[NT / 64];
+  const int i = blockIdx.x;
+  const float* xr = x + (rows ? rows[i] : (long long)i) * d;
+  float sq = 0.f;
+  for (int c = threadIdx.x; c < d; c += NT) sq += xr[c] * xr[c];
+  const float r = 1.f / sqrtf(block_sum<NT>(sq, scratch) / (float)d + eps);
+  for (int c = threadIdx.x; c < d; c += NT) out[(long long)i * d + c] = (T)(xr[c] * r * (offset + w[c]));
+}
+
+template <typename T>
+__global__ __launch_bounds__(NT) void residual_mix_norm_kernel(ResidualMixArgs a) {
+  __shared__ float scratch[NT / 64];
+  const int row = blockIdx.x, d = a.d;
+  float* xr = a.x + (long long)row * d;
+  const long long o = (long long)row * d;
+  float sq = 0.f;
+  for (int c = threadIdx.x; c < d; c += NT) {
+    float s = ldf(a.a, a.a_f32, o + c);
+    if (a.bias_a) s += a.bias_a[c];
+    s *= a.sa;
+    if (a.b) s += a.sb * ldf(a.b, a.b_f32, o + c);
+    if (a.c) s += a.sc * ldf(a.c, a.c_f32, o + c);
+    const float xn = xr[c] + s;
+    xr[c] = xn;
+    sq += xn * xn;
+  }
+  if (!a.out) return;
+  const float r = 1.f / sqrtf(block_sum<NT>(sq, scratch) / (float)d + a.eps);
+  T* out = reinterpret_cast<T*>(a.out) + o;
+  // (each thread re-reads the columns it wrote itself)
+  for (int c = threadIdx.x; c < d; c += NT) out[c] = (T)(xr[c] * r * (a.offset + a.w[c]));
+}
+
+template <typename T>
+__global__ __launch_bounds__(NT) void qkv_rope_cache_kernel(QkvRopeArgs a) {
+  const int row = blockIdx.x;
+  const T* z = reinterpret_cast<const T*>(a.z) + (long long)row * a.ldz;
+  const int nq = a.H * a.dk, nk = a.G * a.dk, nv = a.G * a.dv;
+  const int rot = 2 * a.pairs;
+  const float* cs = a.rope + (long long)a.positions[row] * rot;   // [pairs][2]
+  const int slot = a.slots[row];
+  T* qo = reinterpret_cast<T*>(a.q_out) + (long long)row * nq;
+  T* kc = slot >= 0 ? reinterpret_cast<T*>(a.k_cache) + (long long)slot * nk : nullptr;
+  T* vc = slot >= 0 ? reinterpret_cast<T*>(a.v_cache) + (long long)slot * nv : nullptr;
+  for (int i = threadIdx.x; i < nq + nk; i += NT) {
+    const int e = i < nq ? i % a.dk : (i - nq) % a.dk;   // entry within its head
+    float v = (float)z[i] + a.bias[i];
+    if (e < rot) {
+      const int j = i - e + (e ^ 1);                     // the pair's other entry
+      const float u = (float)z[j] + a.bias[j];
+      const float c = cs[e & ~1], s = cs[(e & ~1) + 1];
+      v = (e & 1) ? v * c + u * s : v * c - u * s;
+    }
+    if (i < nq) qo[i] = (T)v;
+    else if (kc) kc[i - nq] = (T)v;
+  }
+  if (vc)
+    for (int i = threadIdx.x; i < nv; i += NT) vc[i] = (T)((float)z[nq + nk + i] + a.bias[nq + nk + i]);
+}
+
+// grid (T, C / group); BT threads over the group's columns
+template <typename T, int BT>
+__global__ __launch_bounds__(BT) void gated_group_norm_kernel(const float* __restrict__ y, const T* __restrict__ gate,
+                                                              long long ldg, const float* __restrict__ w, int wlen,
+                                                              float eps, int group, int gate_first, T* __restrict__ out,
+                                                              int C) {
+  __shared__ float scratch[BT / 64];
+  const int row = blockIdx.x, c0 = blockIdx.y * group;
+  const float* yr = y + (long long)row * C + c0;
+  const T* gr = gate + (long long)row * ldg + c0;
+  float sq = 0.f;
+  for (int c = threadIdx.x; c < group; c += BT) {
+    float v = yr[c];
+    if (gate_first) v *= silu_exact((float)gr[c]);
+    sq += v * v;
+  }
+  const float r = 1.f / sqrtf(block_sum<BT>(sq, scratch) / (float)group + eps);
+  T* orow = out + (long long)row * C + c0;
+  for (int c = threadIdx.x; c < group; c += BT) {
+    const float g = silu_exact((float)gr[c]);
+    const float wv = w[(c0 + c) % wlen];
+    orow[c] = (T)(gate_first ? yr[c] * g * r * wv : yr[c] * r * wv * g);
+  }
+}
+
+// grid (T, ceil(C / NT)): one thread per (row, channel)
+template <typename T>
+__global__ __launch_bounds__(NT) void causal_conv_silu_kernel(ConvArgs a) {
+  const int row = blockIdx.x, c = blockIdx.y * NT + threadIdx.x;
+  if (c >= a.C) return;
+  const int s0 = a.cu_q ? a.cu_q[a.row_seq[row]] : row;
+  const int j = row - s0, taps = a.taps;
+  const int pr = a.prev_row[s0];
+  const T* st = pr <= -2 ? reinterpret_cast<const T*>(a.state) + (long long)(-(pr + 2)) * a.state_stride : nullptr;
+  const T* x = reinterpret_cast<const T*>(a.xin);
+  const T* w = reinterpret_cast<const T*>(a.w) + (long long)c * taps;
+  float acc = a.b[c];
+  for (int i = 0; i < taps; ++i) {       // i positions back
+    float v = 0.f;
+    if (i <= j) v = (float)x[(long long)(row - i) * a.ldx + c];
+    else if (st) v = (float)st[(long long)(taps - 1 - (i - j)) * a.C + c];
+    acc += (float)w[taps - 1 - i] * v;
+  }
+  reinterpret_cast<T*>(a.out)[(long long)row * a.C + c] = (T)(acc * sigmoidf(acc));
+}
+
+constexpr int MAX_TAPS = 16;
+
+// grid (runs, ceil(C / NT)): one thread per (run, channel) owns that channel of the run's state slot
+template <typename T>
+__global__ __launch_bounds__(NT) void conv_state_update_kernel(ConvArgs a) {
+  const int run = blockIdx.x, c = blockIdx.y * NT + threadIdx.x;
+  if (c >= a.C) return;
+  const int s0 = a.cu_q ? a.cu_q[run] : run, s1 = a.cu_q ? a.cu_q[run + 1] : run + 1;
+  if (s1 <= s0) return;
+  const int sv = a.save_slot[s1 - 1];
+  if (sv < 0) return;
+  const int keep = a.taps - 1, n = s1 - s0;
+  const int pr = a.prev_row[s0];
+  T* base = reinterpret_cast<T*>(a.state);
+  const T* old = pr <= -2 ? base + (long long)(-(pr + 2)) * a.state_stride : nullptr;
+  const T* x = reinterpret_cast<const T*>(a.xin);
+  T vals[MAX_TAPS];
+#pragma unroll
+  for (int m = 0; m < MAX_TAPS; ++m) {
+    if (m < keep) {
+      const int back = keep - m;       // 1 = the newest input
+      T v = (T)0.f;
+      if (back <= n) v = x[(long long)(s1 - back) * a.ldx + c];
+      else if (old) v = old[(long long)(keep - (back - n)) * a.C + c];
+      vals[m] = v;
+    }
+  }
+  T* dst = base + (long long)sv * a.state_stride;
+#pragma unroll
+  for (int m = 0; m < MAX_TAPS; ++m)
+    if (m < keep) dst[(long long)m * a.C + c] = vals[m];
+}
+
+template <typename T>
+__global__ __launch_bounds__(NT) void relu_sq_kernel(const T* __restrict__ a, long long lda, T* __restrict__ out, int R,
+                                                     int F) {
+  const long long n = (long long)R * F;
+  for (long long i = (long long)blockIdx.x * NT + threadIdx.x; i < n; i += (long long)gridDim.x * NT) {
+    const long long r = i / F, c = i - r * F;
+    const float v = fmaxf((float)a[r * lda + c], 0.f);
+    out[i] = (T)(v * v);
+  }
+}
+
+template <typename T>
+__global__ __launch_bounds__(NT) void silu_mul_kernel(const T* __restrict__ g, long long ldg, const T* __restrict__ u,
+                                                      long long ldu, T* __restrict__ out, int R, int F) {
+  const long long n = (long long)R * F;
+  for (long long i = (long long)blockIdx.x * NT + threadIdx.x; i < n; i += (long long)gridDim.x * NT) {
+    const long long r = i / F, c = i - r * F;
+    const float gv = (float)g[r * ldg + c];
+    out[i] = (T)(gv * sigmoidf(gv) * (float)u[r * ldu + c]);
+  }
+}
+
+// One workgroup per token: the four waves share the router outputs (a wave per output, lanes over the width), then the
+// first wave normalises and picks.  Dynamic LDS: En floats.
+template <typename T>
+__global__ __launch_bounds__(NT) void softmax_topk_kernel(const T* __restrict__ x, const T* __restrict__ Wr,
+                                                          const float* __restrict__ corr, int d, int En, int k,
+                                                          int* __restrict__ ids, float* __restrict__ w) {
+  extern __shared__ float sc[];
+  const int t = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const T* xr = x + (long long)t * d;
+  for (int e = wave; e < En; e += NT / 64) {
+    const T* wr = Wr + (long long)e * d;
+    float acc = 0.f;
+    for (int c = lane; c < d; c += 64) acc += (float)xr[c] * (float)wr[c];
+    acc = wave_sum(acc);
+    if (lane == 0) sc[e] = acc;
+  }
+  __syncthreads();
+  if (wave == 0) {
+    float m = -INFINITY;
+    for (int e = lane; e < En; e += 64) m = fmaxf(m, sc[e]);
+    m = wave_max(m);
+    float sum = 0.f;
+    for (int e = lane; e < En; e += 64) sum += expf(sc[e] - m);
+    sum = wave_sum(sum);
+    const float inv = 1.f / sum;
+    for (int e = lane; e < En; e += 64) sc[e] = expf(sc[e] - m) * inv;   // (each lane rewrites the entries it read)
+  }
+  __syncthreads();
+  if (wave) return;
+  unsigned long long taken = 0;   // bit i: this lane's entry lane + 64 i is chosen (En <= 4096)
+  for (int j = 0; j < k; ++j) {
+    float best = -INFINITY;
+    int bi = 0x7fffffff;
+    for (int e = lane, i = 0; e < En; e += 64, ++i) {
+      if ((taken >> i) & 1) continue;
+      const float v = sc[e] + corr[e];
+      if (v > best) { best = v; bi = e; }     // ascending e: the lowest index wins a tie within the lane
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+      const float ob = __shfl_xor(best, o, 64);
+      const int oi = __shfl_xor(bi, o, 64);
+      if (ob > best || (ob == best && oi < bi)) { best = ob; bi = oi; }
+    }
+    if (bi >= En) bi = j;   // only with non-finite scores: keep the id a valid segment index for the kernels downstream
+    if ((bi & 63) == lane) taken |= 1ull << (bi >> 6);
+    if (lane == 0) {
+      ids[(long long)t * k + j] = bi;
+      w[(long long)t * k + j] = sc[bi];
+    }
+  }
+}
+
+template <typename T>
+__global__ __launch_bounds__(NT) void moe_mix_kernel(const T* __restrict__ y, const int* __restrict__ dst,
+                                                     const int* __restrict__ ids, const float* __restrict__ w, int k, int E,
+                                                     const T* __restrict__ h, const T* __restrict__ shared,
+                                                     const T* __restrict__ sgate, long long ldsg, float* __restrict__ out,
+                                                     int d) {
+  const int t = blockIdx.x;
+  const float sg = shared ? sigmoidf((float)sgate[(long long)t * ldsg]) : 0.f;
+  for (int c = threadIdx.x; c < d; c += NT) {
+    float acc = 0.f;
+    for (int j = 0; j < k; ++j) {
+      const long long a = (long long)t * k + j;
+      const float v = ids[a] >= E ? (float)h[(long long)t * d + c] : (float)y[(long long)dst[a] * d + c];
+      acc += w[a] * v;
+    }
+    if (shared) acc += sg * (float)shared[(long long)t * d + c];
+    out[(long long)t * d + c] = acc;
+  }
+}
+
+int ew_grid(long long n) {
+  long long g = (n + NT - 1) / NT;
+  return (int)(g < 1 ? 1 : (g > 16384 ? 16384 : g));
+}
+
+}  // namespace
+
+#define DISPATCH_T(f32, ...)            \
+  if (f32) {                            \
+    using T = float;                    \
+    __VA_ARGS__                         \
+  } else {                              \
+    using T = bf16;                     \
+    __VA_ARGS__                         \
+  }
+
+void launch_embed_norm(const int* ids, const int* src, const int* prev, const void* table, const float* w, float eps,
+                       float offset, float* x, int T_, int d, int f32, hipStream_t s) {
+  if (T_ <= 0) return;
+  DISPATCH_T(f32, embed_norm_kernel<T><<<T_, NT, 0, s>>>(ids, src, prev, (const T*)table, w, eps, offset, x, d);)
+}
+
+void launch_rms_norm_rows(const float* x, const long long* rows, const float* w, float eps, float offset, void* out,
+                          int n, int d, int f32, hipStream_t s) {
+  if (n <= 0) return;
+  DISPATCH_T(f32, rms_norm_rows_kernel<T><<<n, NT, 0, s>>>(x, rows, w, eps, offset, (T*)out, d);)
+}
+
+void launch_residual_mix_norm(const ResidualMixArgs& a, int f32, hipStream_t s) {
+  if (a.T <= 0) return;
+  DISPATCH_T(f32, residual_mix_norm_kernel<T><<<a.T, NT, 0, s>>>(a);)
+}
+
+void launch_qkv_rope_cache(const QkvRopeArgs& a, int T_, int f32, hipStream_t s) {
+  if (T_ <= 0) return;
+  DISPATCH_T(f32, qkv_rope_cache_kernel<T><<<T_, NT, 0, s>>>(a);)
+}
+
+void launch_gated_group_norm(const float* y, const void* gate, long long ldg, const float* w, int wlen, float eps,
+                             int group, int gate_first, void* out, int T_, int C, int f32, hipStream_t s) {
+  if (T_ <= 0) return;
+  dim3 grid(T_, C / group);
+  if (group <= 256) {
+    DISPATCH_T(f32, (gated_group_norm_kernel<T, 64><<<grid, 64, 0, s>>>(y, (const T*)gate, ldg, w, wlen, eps, group,
+                                                                          gate_first, (T*)out, C));)
+  } else {
+    DISPATCH_T(f32, (gated_group_norm_kernel<T, NT><<<grid, NT, 0, s>>>(y, (const T*)gate, ldg, w, wlen, eps, group,
+                                                                          gate_first, (T*)out, C));)
+  }
+}
+
+void launch_causal_conv_silu(const ConvArgs& a, int f32, hipStream_t s) {
+  if (a.T <= 0) return;
+  dim3 grid(a.T, (a.C + NT - 1) / NT);
+  DISPATCH_T(f32, causal_conv_silu_kernel<T><<<grid, NT, 0, s>>>(a);)
+}
+
+void launch_conv_state_update(const ConvArgs& a, int f32, hipStream_t s) {
+  if (a.runs <= 0 || a.taps <= 1) return;
+  dim3 grid(a.runs, (a.C + NT - 1) / NT);
+  DISPATCH_T(f32, conv_state_update_kernel<T><<<grid, NT, 0, s>>>(a);)
+}
+
+void launch_relu_sq(const void* a, long long lda, void* out, int R, int F, int f32, hipStream_t s) {
+  if (R <= 0) return;
+  DISPATCH_T(f32, relu_sq_kernel<T><<<ew_grid((long long)R * F), NT, 0, s>>>((const T*)a, lda, (T*)out, R, F);)
+}
+
+void launch_silu_mul(const void* gate, long long ldg, const void* up, long long ldu, void* out, int R, int F, int f32,
+                     hipStream_t s) {
+  if (R <= 0) return;
+  DISPATCH_T(f32, silu_mul_kernel<T><<<ew_grid((long long)R * F), NT, 0, s>>>((const T*)gate, ldg, (const T*)up, ldu,
+                                                                              (T*)out, R, F);)
+}
+
+void launch_softmax_topk(const void* x, const void* Wr, const float* corr, int T_, int d, int En, int k, int* ids,
+                         float* w, int f32, hipStream_t s) {
+  if (T_ <= 0) return;
+  DISPATCH_T(f32, softmax_topk_kernel<T><<<T_, NT, En * sizeof(float), s>>>((const T*)x, (const T*)Wr, corr, d, En, k,
+                                                                            ids, w);)
+}
+
+void launch_moe_mix(const void* y, const int* dst, const int* ids, const float* w, int k, int E, const void* h,
+                    const void* shared, const void* sgate, long long ldsg, float* out, int T_, int d, int f32,
+                    hipStream_t s) {
+  if (T_ <= 0) return;
+  DISPATCH_T(f32, moe_mix_kernel<T><<<T_, NT, 0, s>>>((const T*)y, dst, ids, w, k, E, (const T*)h, (const T*)shared,
+                                                     (const T*)sgate, ldsg, out, d);)
+}

@@ -46,6 +46,13 @@ LATENT_SO = os.path.join(PKG, "_C_latent.so")
 # their own, so a process that serves only such a model builds (and loads) these three translation units
 LATENT_KERNELS = ("seq_mix.hip", "latent_attention.hip", "glu_moe.hip")
 LATENT_BINDINGS = ("latent_ops.cpp",)
+# the kernels of the hybrid family (windowed attention, decaying linear recurrences, carried convolutions, parallel
+# feed-forward with a softmax router) and their op bindings; the routed feed-forward shares glu_moe.hip's expert-segment
+# kernels, so that translation unit is linked into both libraries
+HYBRID_SO = os.path.join(PKG, "_C_hybrid.so")
+HYBRID_KERNELS = ("hybrid_rows.hip", "window_attention.hip", "decay_scan.hip")
+HYBRID_SHARED = ("glu_moe.hip",)
+HYBRID_BINDINGS = ("hybrid_ops.cpp",)
 NET_SO = os.path.join(PKG, "net", "_native.so")
 RUNTIME_SO = os.path.join(PKG, "runtime", "_runtime.so")
 
@@ -104,7 +111,7 @@ def build_kernels(verbose: bool = False, force: bool = False) -> str:
     os.makedirs(OBJ, exist_ok=True)
     kdir = os.path.join(CSRC, "kernels")
     headers = glob.glob(os.path.join(kdir, "*.h")) + glob.glob(os.path.join(kdir, "*.cuh"))
-    sources = sorted(s for s in glob.glob(os.path.join(kdir, "*.hip")) if os.path.basename(s) not in LATENT_KERNELS)
+    sources = sorted(s for s in glob.glob(os.path.join(kdir, "*.hip")) if os.path.basename(s) not in LATENT_KERNELS + HYBRID_KERNELS)
     tinc, tlib, abi = _torch_paths()
     jobs = []
     objs = []
@@ -115,7 +122,7 @@ def build_kernels(verbose: bool = False, force: bool = False) -> str:
             cmd = [HIPCC, "-c", src, "-o", obj, "-I", kdir] + HIP_FLAGS
             jobs.append(cmd)
     for bsrc in sorted(b for b in glob.glob(os.path.join(CSRC, "bindings", "*.cpp"))
-                       if os.path.basename(b) not in LATENT_BINDINGS):
+                       if os.path.basename(b) not in LATENT_BINDINGS + HYBRID_BINDINGS):
         bobj = os.path.join(OBJ, "bind_" + os.path.basename(bsrc) + ".o")
         objs.append(bobj)
         if force or _newer(bobj, [bsrc] + headers):
@@ -171,6 +178,41 @@ def build_latent(verbose: bool = False, force: bool = False) -> str:
              verbose)
         os.replace(tmp, LATENT_SO)
     return LATENT_SO
+
+
+def build_hybrid(verbose: bool = False, force: bool = False) -> str:
+    """csrc/kernels/{hybrid_rows,window_attention,decay_scan,glu_moe}.hip + csrc/bindings/hybrid_ops.cpp ->
+    symmetry_amd/_C_hybrid.so (``torch.ops.symmetry_amd_hybrid``)."""
+    os.makedirs(OBJ, exist_ok=True)
+    kdir = os.path.join(CSRC, "kernels")
+    headers = [os.path.join(kdir, h) for h in ("common.h", "hybrid_launchers.h", "latent_launchers.h")]
+    tinc, tlib, abi = _torch_paths()
+    jobs, objs = [], []
+    for name in HYBRID_KERNELS + HYBRID_SHARED:
+        src, obj = os.path.join(kdir, name), os.path.join(OBJ, name + ".o")
+        objs.append(obj)
+        if force or _newer(obj, [src] + headers):
+            jobs.append([HIPCC, "-c", src, "-o", obj, "-I", kdir] + HIP_FLAGS + NO_PACKED_FP32)
+    for name in HYBRID_BINDINGS:
+        src, obj = os.path.join(CSRC, "bindings", name), os.path.join(OBJ, "bind_" + name + ".o")
+        objs.append(obj)
+        if force or _newer(obj, [src] + headers):
+            cmd = [HIPCC, "-c", src, "-o", obj, "-I", kdir, "-O2", "-std=c++17", "-fPIC", f"--offload-arch={ARCH}",
+                   "-D__HIP_PLATFORM_AMD__=1", "-DUSE_ROCM=1", f"-D_GLIBCXX_USE_CXX11_ABI={abi}",
+                   "-DTORCH_EXTENSION_NAME=_C_hybrid", "-Wno-unused-result", "-Wno-deprecated-declarations"]
+            for i in tinc:
+                cmd += ["-isystem", i]
+            jobs.append(cmd)
+    if jobs:
+        with cf.ThreadPoolExecutor(_jobs()) as ex:
+            list(ex.map(lambda c: _run(c, verbose), jobs))
+    if force or jobs or _newer(HYBRID_SO, objs):
+        tmp = HYBRID_SO + f".{os.getpid()}.tmp"  # atomic: two first-use builds may race
+        _run([HIPCC, "-shared", "-o", tmp] + objs + [f"--offload-arch={ARCH}", "-L", tlib, "-lc10", "-lc10_hip",
+                                                      "-ltorch_cpu", "-ltorch_hip", "-ltorch", f"-Wl,-rpath,{tlib}"],
+             verbose)
+        os.replace(tmp, HYBRID_SO)
+    return HYBRID_SO
 
 
 # --------------------------------------------------------------------------------------
@@ -251,6 +293,7 @@ def build_all(verbose: bool = False, force: bool = False):
     build_runtime(verbose, force)
     ker = build_kernels(verbose, force)
     build_latent(verbose, force)
+    build_hybrid(verbose, force)
     return ker, net
 
 
@@ -264,6 +307,8 @@ if __name__ == "__main__":
         print(build_kernels(verbose, force))
     if not what or "latent" in what:
         print(build_latent(verbose, force))
+    if not what or "hybrid" in what:
+        print(build_hybrid(verbose, force))
     if not what or "runtime" in what:
         print(build_runtime(verbose, force))
     if "selftest" in what:

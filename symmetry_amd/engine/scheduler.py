@@ -405,6 +405,8 @@ class Scheduler:
         for seq, n, offs in entries:
             if n <= 0 or seq.num_computed + n > seq.num_tokens:
                 raise ValueError(f"{seq.request_id}: {n} tokens past its {seq.num_tokens - seq.num_computed} known ones")
+            if any(o < 0 or o >= n for o in offs):
+                raise ValueError(f"{seq.request_id}: wanted offsets {list(offs)} outside this step's {n} tokens")
             if seq not in self.running:
                 if len(self.running) >= self.cfg.max_num_seqs or (self.slots is not None and not self.slots.alloc(seq)):
                     raise MemoryError(f"{seq.request_id}: no free sequence slot ({self.cfg.max_num_seqs} live)")

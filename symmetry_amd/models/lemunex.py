@@ -287,7 +287,7 @@ class LemunexLM:
         cu = b.cu_q if b.kind != "decode" else None
         xin = self._cols(z, P, "xbc")
         xc = self._buf("ssm.xc", (T, m.conv_channels))
-        ops.causal_conv_silu(xin, P["conv"], P["conv.b"], cache.conv[i], cu, b.prev_row, runs, xc)
+        ops.causal_conv_silu(xin, P["conv"], P["conv.b"], cache.conv[i], cu, b.row_seq, b.prev_row, runs, xc)
         ops.conv_state_update(xin, cache.conv[i], cu, b.prev_row, b.save_slot, runs)
         inner, gn = m.inner, m.groups * m.state
         y = self._buf("rec.y", (T, inner), torch.float32)

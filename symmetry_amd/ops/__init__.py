@@ -755,18 +755,21 @@ def qkv_rope_cache(z, bias, H, G, dk, dv, positions, slots, rope, q_out, k_cache
     return reference.qkv_rope_cache(z, bias, H, G, dk, dv, positions, slots, rope, q_out, k_cache, v_cache)
 
 
-WINDOW_ATTN_IMPL = os.environ.get("SYMMETRY_WINDOW_ATTN", "auto")
+WINDOW_ATTN_IMPL = 0 if os.environ.get("SYMMETRY_WINDOW_ATTN", "auto") == "wave" else 1  # A/B: the all-shapes kernel
 
 
-def window_attn(q, k_cache, v_cache, block_tables, row_seq, positions, window, scale, gate, out, tiles=None, cu_q=None):
+def window_attn(q, k_cache, v_cache, block_tables, row_seq, positions, window, scale, gate, out, tiles=None, cu_q=None,
+                impl=None):
     """Softmax attention of q [T, H, dk] over the paged caches: row r sees positions max(0, p - window + 1) .. p of
     sequence row_seq[r] (p = positions[r]); query head h reads key / value head h // (H / G); scores and weights
     fp32.  ``gate`` [T, H] (a view): head outputs are multiplied by sigmoid(gate).  ``tiles`` / ``cu_q``: the packed
-    prompt form (64-row query tiles), for the tiled kernel."""
+    prompt form (64-row query tiles), for the tiled kernel.  Returns the implementation used (0: one wave per (row,
+    head), every shape; 1: tiled)."""
     if _gpu(q):
         return _hyb().window_attn(q, k_cache, v_cache, block_tables, row_seq, positions, int(window), float(scale), gate,
-                                  out, tiles, cu_q)
-    return reference.window_attn(q, k_cache, v_cache, block_tables, row_seq, positions, window, scale, gate, out)
+                                  out, tiles, cu_q, WINDOW_ATTN_IMPL if impl is None else int(impl))
+    reference.window_attn(q, k_cache, v_cache, block_tables, row_seq, positions, window, scale, gate, out)
+    return 0
 
 
 DECAY_CHANNEL_GATE, DECAY_STEP_SIZE = 0, 1
@@ -797,11 +800,12 @@ def gated_group_norm(y, gate, w, eps, group, gate_first, out):
     return reference.gated_group_norm(y, gate, w, eps, group, gate_first, out)
 
 
-def causal_conv_silu(xin, w, b, state, cu_q, prev_row, runs, out):
+def causal_conv_silu(xin, w, b, state, cu_q, row_seq, prev_row, runs, out):
     """out_t = silu(b + sum_j w[:, taps - 1 - j] x_(t - j)) per channel over every run; inputs before the run come from
     state[slot] [taps - 1, C] (prev_row[first] <= -2) or are zero.  xin [T, C] (view)."""
     if _gpu(out):
-        return _hyb().causal_conv_silu(xin, w, b, state, cu_q, prev_row, int(runs), out)
+        return _hyb().causal_conv_silu(xin, w, b, state, cu_q, row_seq if cu_q is not None else None, prev_row, int(runs),
+                                       out)
     return reference.causal_conv_silu(xin, w, b, state, cu_q, prev_row, runs, out)
 
 

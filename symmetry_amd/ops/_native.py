@@ -77,3 +77,27 @@ def latent_ops():
 
 def latent_library_path() -> str:
     return _LATENT_LIB
+
+
+# ---- the hybrid family's kernels (windowed attention, decaying recurrences, carried convolutions): _C_hybrid.so ------
+_HYBRID_LIB = os.path.join(os.path.dirname(_LIB), "_C_hybrid.so")
+_hybrid_loaded = False
+
+
+def hybrid_ops():
+    """``torch.ops.symmetry_amd_hybrid`` (loaded once; built first if the library is missing: five translation units,
+    under a minute).  Raises if it cannot be built or loaded: no eager fallback on the device."""
+    global _hybrid_loaded
+    with _lock:
+        if not _hybrid_loaded:
+            if not os.path.exists(_HYBRID_LIB):
+                from symmetry_amd import _build
+
+                _build.build_hybrid()
+            torch.ops.load_library(_HYBRID_LIB)
+            _hybrid_loaded = True
+    return torch.ops.symmetry_amd_hybrid
+
+
+def hybrid_library_path() -> str:
+    return _HYBRID_LIB

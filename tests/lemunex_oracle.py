@@ -168,8 +168,8 @@ def moe_ff(W, p, spec, h, margins=None):
     r = spec["router"]
     E = int(r["experts"])
     idx, wt, margin = route(W, p, spec, h)
-    if margins is not None:
-        margins.append(margin)
+    if margins is not None:   # a near-tie only matters if the expert it may swap in or out carries weight
+        margins.append(torch.where(wt[:, -1] > 0.05, margin, torch.full_like(margin, math.inf)))
     out = torch.zeros_like(h)
     for t in range(h.shape[0]):
         for e, w in zip(idx[t].tolist(), wt[t]):
