@@ -325,6 +325,7 @@ ConvArgs conv_args(const Tensor& xin, const OptTensor& w, const OptTensor& b, Te
     TORCH_CHECK(save_slot->numel() >= T, "conv: save_slot too short");
     a.save_slot = ptr<int>(*save_slot);
   }
+  a.prev_row = ptr<int>(prev_row);
   a.xin = xin.data_ptr();
   a.state = state.data_ptr();
   a.state_stride = state.stride(0);
