@@ -1,5 +1,5 @@
 #!/usr/bin/env python3
-"""Prefill and decode throughput of a Bozevik stack beside the closest Llama / Mixtral stack of equal size.
+"""Prefill and decode throughput of a Bozevik or Lemunex stack beside the closest Llama / Mixtral stack of equal size.
 
 Random weights, layer shapes of real models, a few layers each (throughput per layer is what is compared; the
 vocabulary projection is the same size on both sides).  Per size and family, through the engine's own scheduler:
@@ -40,6 +40,28 @@ def _pairs():
         # routed: 16 experts, 4 per token (+ a shared expert on the Bozevik side; equal active width 6144)
         "moe-w2048": (_bozevik_stack("bozevik-moe", 32768, 2048, 4, heads=16, ff=8192, experts=16, top=4, expert_ff=1024,
                                      shared_ff=2048, share_every=2, moe_every=1, **lat, **kw),
+                      ModelConfig("mixtral-w2048", 32768, 2048, 1536, 4, 16, 4, num_experts=16, top_k=4, **kw)),
+    }
+
+
+def _lemunex_pairs():
+    """Lemunex stacks (attention + linear attention layers around state-space layers) beside the Llama / Mixtral stack of
+    the same width, head count and feed-forward width; the attention window equals the benchmark's prompt length."""
+    from symmetry_amd.models.config import ModelConfig, lemunex_stack
+
+    kw = dict(max_position=8192, bos_token_id=32000, eos_token_ids=(32001, 32002))
+    return {
+        "w2048": (lemunex_stack("lemunex-w2048", 32768, 2048, "pmmp", heads=16, kv_heads=4, dim=128, window=1024,
+                                gla_heads=8, gla_dim=128, gla_vdim=256, ssm_heads=64, ssm_vdim=64, ssm_state=128, ff=8192,
+                                **kw),
+                  ModelConfig("llama-w2048", 32768, 2048, 8192, 4, 16, 4, **kw)),
+        "w4096": (lemunex_stack("lemunex-w4096", 32768, 4096, "pmmp", heads=32, kv_heads=8, dim=128, window=1024,
+                                gla_heads=16, gla_dim=128, gla_vdim=256, ssm_heads=128, ssm_vdim=64, ssm_state=128,
+                                ff=14336, **kw),
+                  ModelConfig("llama-w4096", 32768, 4096, 14336, 4, 32, 8, **kw)),
+        "moe-w2048": (lemunex_stack("lemunex-moe", 32768, 2048, "PMMP", heads=16, kv_heads=4, dim=128, window=1024,
+                                    gla_heads=8, gla_dim=128, gla_vdim=256, ssm_heads=64, ssm_vdim=64, ssm_state=128,
+                                    ff=8192, experts=16, top=4, identity=2, expert_ff=1024, shared_ff=2048, **kw),
                       ModelConfig("mixtral-w2048", 32768, 2048, 1536, 4, 16, 4, num_experts=16, top_k=4, **kw)),
     }
 
@@ -95,22 +117,23 @@ def main(argv=None) -> int:
     ap.add_argument("--prompts", type=int, default=8)
     ap.add_argument("--prompt-len", type=int, default=1024)
     ap.add_argument("--decode-steps", type=int, default=64)
-    ap.add_argument("--only", default="", help="bozevik | baseline: one side only (profiling)")
+    ap.add_argument("--only", default="", help="bozevik | lemunex | baseline: one side only (profiling)")
+    ap.add_argument("--design", default="bozevik", choices=("bozevik", "lemunex"), help="the family measured")
     a = ap.parse_args(argv)
-    pairs = _pairs()
+    pairs = _pairs() if a.design == "bozevik" else _lemunex_pairs()
     ratios = {}
     for size in a.sizes.split(","):
         boz, base = pairs[size]
         rows = {}
-        for side, cfg in (("bozevik", boz), ("baseline", base)):
+        for side, cfg in ((a.design, boz), ("baseline", base)):
             if a.only and a.only != side:
                 continue
             rows[side] = measure(cfg, a.prompts, a.prompt_len, a.decode_steps)
             print(json.dumps({"size": size, "family": side, **rows[side]}), flush=True)
         if len(rows) == 2:
-            ratios[size] = {k: round(rows["bozevik"][k] / rows["baseline"][k], 3) for k in ("prefill_tok_s", "decode_tok_s")}
+            ratios[size] = {k: round(rows[a.design][k] / rows["baseline"][k], 3) for k in ("prefill_tok_s", "decode_tok_s")}
     if ratios:
-        print(json.dumps({"bozevik_over_baseline": ratios}), flush=True)
+        print(json.dumps({a.design + "_over_baseline": ratios}), flush=True)
     return 0
 
 

@@ -5,10 +5,10 @@
 // head h / (H / G).  Key and value head sizes are independent (dk, dv).  Scores, softmax statistics, weights and the
 // weighted sum are fp32.
 //
-// window_attn_wave_kernel: one wave per (row, head), every shape, bf16 or fp32.  The window is walked in tiles of 64
-// keys: each lane scores one key (the query sits in LDS as fp32, the key row is read in 16-byte pieces where the
-// head size allows), the wave forms the tile's running max / sum, then the lanes switch to value columns and add
-// the tile's weighted value rows (weights broadcast from LDS, value rows read coalesced).
+// window_attn_wave_kernel: one to eight waves per (row, head), every shape, bf16 or fp32.  The window is walked in
+// tiles of 64 keys: each lane scores one key (the query sits in LDS as fp32, the key row is read in 16-byte pieces
+// where the head size allows), the wave forms the tile's running max / sum, then the lanes switch to value columns
+// and add the tile's weighted value rows (weights read lane by lane, value rows read coalesced).
 #include "common.h"
 #include "hybrid_launchers.h"
 
@@ -49,19 +49,21 @@ SYM_DEV float dot_row<float>(const float* __restrict__ k, const float* __restric
   return acc;
 }
 
-// grid (H, T), 64 threads.  Dynamic LDS: (dk + 64) floats.
-template <typename T>
-__global__ __launch_bounds__(64) void window_attn_wave_kernel(WindowAttnArgs a) {
+// grid (H, T), NW waves.  Wave w walks the key tiles w, w + NW, ... of the row's window with its own running max / sum /
+// accumulator; the waves' partial results meet in LDS at the end (rows of a decode step have few (row, head) pairs
+// and long windows: NW > 1 shortens each wave's walk).  Dynamic LDS: dk + NW * (2 + 64 * MAX_VCOLS) floats.
+template <typename T, int NW>
+__global__ __launch_bounds__(64 * NW) void window_attn_wave_kernel(WindowAttnArgs a) {
   extern __shared__ float lds[];
-  float* qs = lds;            // [dk]
-  float* ps = lds + a.dk;     // [64]
-  const int h = blockIdx.x, row = blockIdx.y, lane = threadIdx.x;
+  float* qs = lds;                      // [dk]
+  float* part = lds + a.dk;             // [NW][2 + 64 * MAX_VCOLS]: m, l, acc
+  const int h = blockIdx.x, row = blockIdx.y, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int g = h / (a.H / a.G);
   const int p = a.positions[row];
   const int j0 = max(0, p - a.window + 1);
   const int* bt = a.block_tables + (long long)a.row_seq[row] * a.max_blocks;
   const T* q = reinterpret_cast<const T*>(a.q) + ((long long)row * a.H + h) * a.dk;
-  for (int e = lane; e < a.dk; e += 64) qs[e] = (float)q[e] * a.scale;
+  for (int e = threadIdx.x; e < a.dk; e += 64 * NW) qs[e] = (float)q[e] * a.scale;
   __syncthreads();
   const T* kc = reinterpret_cast<const T*>(a.k_cache);
   const T* vc = reinterpret_cast<const T*>(a.v_cache);
@@ -69,7 +71,7 @@ __global__ __launch_bounds__(64) void window_attn_wave_kernel(WindowAttnArgs a) 
 #pragma unroll
   for (int i = 0; i < MAX_VCOLS; ++i) acc[i] = 0.f;
   float m = -INFINITY, l = 0.f;
-  for (int t0 = j0; t0 <= p; t0 += 64) {
+  for (int t0 = j0 + 64 * wave; t0 <= p; t0 += 64 * NW) {
     const int j = t0 + lane;
     float s = -INFINITY;
     if (j <= p) {
@@ -81,9 +83,6 @@ __global__ __launch_bounds__(64) void window_attn_wave_kernel(WindowAttnArgs a) 
     const float corr = expf(m - mt);          // first tile: exp(-inf) = 0 on an all-zero accumulator
     l = l * corr + wave_sum(w);
     m = mt;
-    __syncthreads();                          // the previous tile's weights have been read
-    ps[lane] = w;
-    __syncthreads();
 #pragma unroll
     for (int i = 0; i < MAX_VCOLS; ++i) acc[i] *= corr;
     const int nt = min(64, p - t0 + 1);
@@ -91,12 +90,33 @@ __global__ __launch_bounds__(64) void window_attn_wave_kernel(WindowAttnArgs a) 
       const int jk = t0 + jj;
       const long long slot = (long long)bt[jk / a.BS] * a.BS + jk % a.BS;
       const T* vr = vc + (slot * a.G + g) * a.dv;
-      const float pw = ps[jj];
+      const float pw = __shfl(w, jj, 64);     // (uniform index: a lane read, no LDS)
 #pragma unroll
       for (int i = 0; i < MAX_VCOLS; ++i) {
         const int c = lane + 64 * i;
         if (c < a.dv) acc[i] += pw * (float)vr[c];
       }
+    }
+  }
+  if (NW > 1) {
+    float* mine = part + wave * (2 + 64 * MAX_VCOLS);
+    if (lane == 0) mine[0] = m, mine[1] = l;
+#pragma unroll
+    for (int i = 0; i < MAX_VCOLS; ++i) mine[2 + 64 * i + lane] = acc[i];
+    __syncthreads();
+    if (wave) return;
+    float M = m;
+    for (int w = 1; w < NW; ++w) M = fmaxf(M, part[w * (2 + 64 * MAX_VCOLS)]);
+    const float f0 = expf(m - M);
+    l *= f0;
+#pragma unroll
+    for (int i = 0; i < MAX_VCOLS; ++i) acc[i] *= f0;
+    for (int w = 1; w < NW; ++w) {
+      const float* o = part + w * (2 + 64 * MAX_VCOLS);
+      const float f = expf(o[0] - M);         // a wave without tiles: exp(-inf) = 0
+      l += o[1] * f;
+#pragma unroll
+      for (int i = 0; i < MAX_VCOLS; ++i) acc[i] += o[2 + 64 * i + lane] * f;
     }
   }
   float gate = 1.f;
@@ -113,15 +133,187 @@ __global__ __launch_bounds__(64) void window_attn_wave_kernel(WindowAttnArgs a) 
   }
 }
 
+template <typename T, int NW>
+void launch_wave(const WindowAttnArgs& a, hipStream_t s) {
+  dim3 grid(a.H, a.T);
+  const size_t lds = (size_t)(a.dk + (NW > 1 ? NW * (2 + 64 * MAX_VCOLS) : 0)) * sizeof(float);
+  window_attn_wave_kernel<T, NW><<<grid, 64 * NW, lds, s>>>(a);
+}
+
+// ---- tiled kernel for prompt rows (bf16, head sizes DK = DV in {32, 64, 96, 128}) --------------------------------
+// grid (query tiles, heads), 4 waves.  A tile is 64 consecutive rows of one sequence's run (the runner's tile list);
+// wave w owns rows 16 w .. 16 w + 15.  Keys walk in tiles of 64 from the first position the tile's first row sees to
+// the last row's own position; a key tile's rows go to LDS once for the four waves (keys row-major, values
+// transposed), scores are MFMA products K Q^T (each lane ends up with one query row's scores of four keys per 16-key
+// subtile: the row statistics are two cross-lane steps), the weights go back into the MFMA as bf16 against the
+// transposed values with the keys in the order the score fragments already have.  Statistics, masks and the running
+// rescale are fp32.
+template <int DK, int DV>
+__global__ __launch_bounds__(256) void window_attn_tile_kernel(WindowAttnArgs a) {
+  constexpr int KD = DK / 32, VD = DV / 16, KS = DK + 8, VS = 64 + 8;
+  extern __shared__ __attribute__((aligned(16))) char smem[];
+  bf16* Ks = reinterpret_cast<bf16*>(smem);   // [64][KS]
+  bf16* Vt = Ks + 64 * KS;                    // [DV][VS]
+  const int tile = blockIdx.x, h = blockIdx.y;
+  const int seq = a.tiles[2 * tile], row0 = a.tiles[2 * tile + 1];
+  const int r_hi = a.cu_q[seq + 1], first = a.cu_q[seq] + row0;
+  if (first >= r_hi) return;                  // padding tile (the whole workgroup)
+  const int nrows = min(64, r_hi - first);
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int j = lane & 15, hq = lane >> 4;
+  const int g = h / (a.H / a.G);
+  const int my_row = first + 16 * wave + j;
+  const bool rv = 16 * wave + j < nrows;
+  const int p_first = a.positions[first], p_last = p_first + nrows - 1;
+  const int qp = p_first + 16 * wave + j;
+  const int* bt = a.block_tables + (long long)a.row_seq[first] * a.max_blocks;
+  const bf16* kc = reinterpret_cast<const bf16*>(a.k_cache);
+  const bf16* vc = reinterpret_cast<const bf16*>(a.v_cache);
+  Pack8 qf[KD];
+  {
+    const bf16* q = reinterpret_cast<const bf16*>(a.q) + ((long long)my_row * a.H + h) * DK + 8 * hq;
+#pragma unroll
+    for (int kk = 0; kk < KD; ++kk) {
+      if (rv) qf[kk].u = *reinterpret_cast<const uint4*>(q + 32 * kk);
+      else qf[kk].u = make_uint4(0, 0, 0, 0);
+    }
+  }
+  f32x4 o[VD];
+#pragma unroll
+  for (int i = 0; i < VD; ++i) o[i] = f32x4{0.f, 0.f, 0.f, 0.f};
+  float m = -INFINITY, l = 0.f;
+  const int k_lo = max(0, p_first - a.window + 1);
+  for (int kt = k_lo & ~63; kt <= p_last; kt += 64) {
+    __syncthreads();                          // every wave is done with the previous tile
+    for (int id = threadIdx.x; id < 64 * (DK / 8); id += 256) {
+      const int key = id / (DK / 8), ch = id - key * (DK / 8);
+      const int kp = kt + key;
+      uint4 v = make_uint4(0, 0, 0, 0);
+      if (kp <= p_last) {
+        const long long slot = (long long)bt[kp / a.BS] * a.BS + kp % a.BS;
+        v = *reinterpret_cast<const uint4*>(kc + (slot * a.G + g) * DK + 8 * ch);
+      }
+      *reinterpret_cast<uint4*>(Ks + key * KS + 8 * ch) = v;
+    }
+    for (int id = threadIdx.x; id < 64 * (DV / 8); id += 256) {
+      const int ch = id / 64, key = id - ch * 64;   // consecutive lanes: consecutive keys of one column group
+      const int kp = kt + key;
+      Pack8 v;
+      v.u = make_uint4(0, 0, 0, 0);
+      if (kp <= p_last) {
+        const long long slot = (long long)bt[kp / a.BS] * a.BS + kp % a.BS;
+        v.u = *reinterpret_cast<const uint4*>(vc + (slot * a.G + g) * DV + 8 * ch);
+      }
+#pragma unroll
+      for (int i = 0; i < 8; ++i) Vt[(8 * ch + i) * VS + key] = v.h[i];
+    }
+    __syncthreads();
+    // scores: sc[s][e] = q_j . k_(kt + 16 s + 4 hq + e)
+    float pv[4][4];
+    float mx = -INFINITY;
+#pragma unroll
+    for (int s4 = 0; s4 < 4; ++s4) {
+      f32x4 acc = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int kk = 0; kk < KD; ++kk) {
+        Pack8 kf;
+        kf.u = *reinterpret_cast<const uint4*>(Ks + (16 * s4 + j) * KS + 32 * kk + 8 * hq);
+        acc = mfma16(kf.v, qf[kk].v, acc);
+      }
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const int kp = kt + 16 * s4 + 4 * hq + e;
+        const bool vis = rv && kp <= qp && kp > qp - a.window;
+        pv[s4][e] = vis ? acc[e] * a.scale : -INFINITY;
+        mx = fmaxf(mx, pv[s4][e]);
+      }
+    }
+    mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+    const float mt = fmaxf(m, mx);
+    const float mref = mt == -INFINITY ? 0.f : mt;   // a row that sees nothing yet
+    float sum = 0.f;
+#pragma unroll
+    for (int s4 = 0; s4 < 4; ++s4)
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        pv[s4][e] = __expf(pv[s4][e] - mref);
+        sum += pv[s4][e];
+      }
+    sum += __shfl_xor(sum, 16, 64);
+    sum += __shfl_xor(sum, 32, 64);
+    const float corr = __expf(m - mref);
+    l = l * corr + sum;
+    m = mt;
+#pragma unroll
+    for (int i = 0; i < VD; ++i) o[i] *= corr;
+    // weighted values: key slots of lane group hq in a 32-key chunk c2 are keys 32 c2 + 4 hq + (0..3) and + 16
+#pragma unroll
+    for (int c2 = 0; c2 < 2; ++c2) {
+      Pack8 pf;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        pf.h[e] = (bf16)pv[2 * c2][e];
+        pf.h[4 + e] = (bf16)pv[2 * c2 + 1][e];
+      }
+#pragma unroll
+      for (int cb = 0; cb < VD; ++cb) {
+        const bf16* vrow = Vt + (16 * cb + j) * VS + 32 * c2 + 4 * hq;
+        Pack8 vf;
+        const uint2 lo = *reinterpret_cast<const uint2*>(vrow), hi = *reinterpret_cast<const uint2*>(vrow + 16);
+        vf.u = make_uint4(lo.x, lo.y, hi.x, hi.y);
+        o[cb] = mfma16(vf.v, pf.v, o[cb]);
+      }
+    }
+  }
+  if (!rv) return;
+  float gate = 1.f;
+  if (a.gate) {
+    const float gv = (float)reinterpret_cast<const bf16*>(a.gate)[(long long)my_row * a.ldg + h];
+    gate = 1.f / (1.f + expf(-gv));
+  }
+  const float inv = gate / l;
+  bf16* out = reinterpret_cast<bf16*>(a.out) + ((long long)my_row * a.H + h) * DV + 4 * hq;
+#pragma unroll
+  for (int cb = 0; cb < VD; ++cb) {
+    bf16x4 w4;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) w4[e] = (bf16)(o[cb][e] * inv);
+    *reinterpret_cast<bf16x4*>(out + 16 * cb) = w4;
+  }
+}
+
+template <int D>
+void launch_tile(const WindowAttnArgs& a, hipStream_t s) {
+  dim3 grid(a.ntiles, a.H);
+  const size_t lds = (size_t)(64 * (D + 8) + D * (64 + 8)) * sizeof(bf16);
+  window_attn_tile_kernel<D, D><<<grid, 256, lds, s>>>(a);
+}
+
 }  // namespace
 
 int launch_window_attn(const WindowAttnArgs& a, int f32, int impl, hipStream_t s) {
   if (a.T <= 0) return 0;
-  dim3 grid(a.H, a.T);
-  const size_t lds = (size_t)(a.dk + 64) * sizeof(float);
-  if (f32)
-    window_attn_wave_kernel<float><<<grid, 64, lds, s>>>(a);
-  else
-    window_attn_wave_kernel<bf16><<<grid, 64, lds, s>>>(a);
+  if (impl == 1 && !f32 && a.tiles && a.cu_q && a.ntiles > 0 && a.dk == a.dv && a.ntiles <= 65535 * 16) {
+    switch (a.dk) {
+      case 32: launch_tile<32>(a, s); return 1;
+      case 64: launch_tile<64>(a, s); return 1;
+      case 96: launch_tile<96>(a, s); return 1;
+      case 128: launch_tile<128>(a, s); return 1;
+      default: break;
+    }
+  }
+  // few (row, head) pairs and a long window (decode steps): several waves per pair
+  const long long pairs = (long long)a.T * a.H;
+  const int nw = pairs >= 8192 || a.window <= 128 ? 1 : (a.window <= 512 || pairs >= 2048 ? 4 : 8);
+  if (f32) {
+    if (nw == 1) launch_wave<float, 1>(a, s);
+    else if (nw == 4) launch_wave<float, 4>(a, s);
+    else launch_wave<float, 8>(a, s);
+  } else {
+    if (nw == 1) launch_wave<bf16, 1>(a, s);
+    else if (nw == 4) launch_wave<bf16, 4>(a, s);
+    else launch_wave<bf16, 8>(a, s);
+  }
   return 0;
 }

@@ -300,25 +300,27 @@ def test_rotary_table_and_window_attention(device):
     say("op window_attn", device)
     torch.manual_seed(0)
     for (H, G, dk, dv, win, rot, scaling, n) in [(4, 2, 24, 8, 5, 8, True, 37), (6, 1, 10, 12, 70, 10, False, 90),
-                                                  (8, 2, 32, 32, 33, 16, True, 100), (2, 2, 7, 3, 1, 2, True, 9)]:
+                                                  (8, 2, 32, 32, 33, 16, True, 100), (2, 2, 7, 3, 1, 2, True, 9),
+                                                  (2, 1, 16, 24, 300, 8, True, 330), (2, 2, 8, 70, 600, 4, False, 640)]:
         spec = {"heads": H, "kv_heads": G, "dim": dk, "vdim": dv, "mask": {"size": win}, "scale": 0.41,
                 "rot": {"base": 77.0, "dims": rot}}
         if scaling:
             spec["rot"]["scaling"] = {"factor": 5.0, "original": 50, "fast": 6.0, "slow": 0.5}
         d = 20
-        W = {"q": torch.randn(H * dk, d), "k": torch.randn(G * dk, d) * 2, "v": torch.randn(G * dv, d), "g": torch.randn(H, d),
+        W = {"q": torch.randn(H * dk, d) * 0.3, "k": torch.randn(G * dk, d) * 0.5, "v": torch.randn(G * dv, d), "g": torch.randn(H, d),
              "q.b": torch.randn(H * dk), "k.b": torch.randn(G * dk), "v.b": torch.randn(G * dv),
              "o": torch.eye(H * dv), "o.b": torch.zeros(H * dv)}
         W = {k: v.double() for k, v in W.items()}
         h = torch.randn(n, d).double()
         want = O.window_attention(W, "", spec, h).float()
         r = spec["rot"].get("scaling", {})
-        table = ops.rope_scaled_table(128, rot, 77.0, r.get("factor", 0.0), r.get("original", 0.0), r.get("fast", 0.0),
+        table = ops.rope_scaled_table(n, rot, 77.0, r.get("factor", 0.0), r.get("original", 0.0), r.get("fast", 0.0),
                                       r.get("slow", 0.0))
         z = torch.cat([h @ W["q"].T, h @ W["k"].T, h @ W["v"].T, h @ W["g"].T], 1).float()
         bias = torch.cat([W["q.b"], W["k.b"], W["v.b"]]).float()
-        BS, NB = 8, 16
-        bt = torch.tensor([[3, 9, 1, 7, 12, 4, 10, 2, 15, 6, 11, 5, 0, 0, 0, 0]], dtype=torch.int32)
+        BS = 8
+        NB = n // BS + 3
+        bt = (torch.randperm(NB - 1, generator=torch.Generator().manual_seed(n))[None] + 1).int()   # block 0 stays unused
         pos = torch.arange(n, dtype=torch.int32)
         slots = (bt[0][(pos // BS).long()] * BS + pos % BS).int()
         kc, vc = torch.zeros(NB, BS, G, dk), torch.zeros(NB, BS, G, dv)
@@ -329,6 +331,44 @@ def test_rotary_table_and_window_attention(device):
         row_seq = torch.zeros(n, dtype=torch.int32, device=device)
         ops.window_attn(q, kc, vc, bt, row_seq, pos, win, 0.41, z[:, nq:], out)
         assert torch.allclose(out.cpu().reshape(n, -1), want, atol=2e-4, rtol=2e-4), (H, G, dk, dv, win)
+
+
+@pytest.mark.gpu
+def test_window_attention_tiled_against_wave():
+    """The tiled (MFMA) prompt kernel against the one-wave kernel on the same paged cache: several runs of unequal length
+    that continue earlier context, windows shorter and longer than a key tile, heads sharing key / value heads."""
+    say("op window tiled")
+    torch.manual_seed(3)
+    dev = "cuda"
+    for (H, G, D, win, BS) in [(4, 2, 32, 40, 16), (8, 2, 96, 72, 64), (2, 1, 128, 1000, 64), (6, 6, 64, 5, 16)]:
+        runs = [(0, 130), (37, 64), (200, 1), (64, 65), (5, 200)]          # (tokens already cached, new rows)
+        NBs = [-(-(c + n) // BS) for c, n in runs]
+        NB = sum(NBs) + 1
+        perm = (torch.randperm(NB - 1) + 1).int()
+        bt = torch.zeros(len(runs), max(NBs), dtype=torch.int32)
+        o = 0
+        for i, nb in enumerate(NBs):
+            bt[i, :nb] = perm[o:o + nb]
+            o += nb
+        kc = torch.randn(NB, BS, G, D).bfloat16()
+        vc = torch.randn(NB, BS, G, D).bfloat16()
+        pos, row_seq, cu, tiles = [], [], [0], []
+        for i, (c, n) in enumerate(runs):
+            pos += list(range(c, c + n))
+            row_seq += [i] * n
+            cu.append(cu[-1] + n)
+            tiles += [(i, r) for r in range(0, n, 64)]
+        T_ = len(pos)
+        q = (torch.randn(T_, H, D) * 0.5).bfloat16()
+        gate = torch.randn(T_, H + 2).bfloat16()
+        ti = lambda v: torch.tensor(v, dtype=torch.int32, device=dev)
+        args = [q.to(dev), kc.to(dev), vc.to(dev), bt.to(dev), ti(row_seq), ti(pos)]
+        out = [torch.empty(T_, H, D, dtype=torch.bfloat16, device=dev) for _ in range(2)]
+        g = gate.to(dev)[:, 1:H + 1]
+        used = [ops.window_attn(*args, win, D ** -0.5, g, out[0], ti(tiles), ti(cu), impl=1),
+                ops.window_attn(*args, win, D ** -0.5, g, out[1], None, None, impl=0)]
+        assert used == [1, 0]
+        assert torch.allclose(out[0].float(), out[1].float(), atol=0.02, rtol=0.02), (H, G, D, win)
 
 
 @pytest.mark.parametrize("device", DEVICES)
