@@ -191,7 +191,7 @@ int64_t window_attn(const Tensor& q, const Tensor& k_cache, const Tensor& v_cach
   TORCH_CHECK(k_cache.size(3) == a.dk && v_cache.size(0) == k_cache.size(0) && v_cache.size(1) == a.BS &&
                   v_cache.size(2) == a.G && a.G > 0 && a.H % a.G == 0 && a.dv <= 512 && a.dk <= 4096 && window >= 1 &&
                   out.numel() == (int64_t)a.T * a.H * a.dv && row_seq.numel() >= a.T && positions.numel() >= a.T &&
-                  a.T <= 65535,
+                  a.T <= 65535 && k_cache.size(0) * k_cache.size(1) < (1LL << 31),
               "window_attn: shapes");
   if (gate.has_value()) {
     a.ldg = view2(*gate, f32, a.T, a.H, "gate");

@@ -14,28 +14,31 @@
 // lanes are 16 columns x 4 slices of the key channels, so a lane keeps N / 4 state entries of one column in
 // registers and a token's output is a 4-lane sum (two cross-lane adds).  The per-token vectors that all columns
 // share (q, k, the decays) are staged through LDS for CH tokens at a time by the whole workgroup, with the
-// transcendental part of the decay evaluated once per (token, channel) there.
+// transcendental part of the decay evaluated once per (token, channel) there; the next round's global loads are in
+// flight while the current round is computed (two LDS buffers, one barrier per round).
 #include "common.h"
 #include "hybrid_launchers.h"
 
 namespace {
 
 constexpr int NT = 256;
-constexpr int CH = 8;       // tokens staged per round
 constexpr int PCOLS = 16;   // value columns per wave
 constexpr int SLICES = 4;   // key-channel slices per column (lanes)
 
 SYM_DEV float softplus_exact(float v) { return fmaxf(v, 0.f) + log1pf(expf(-fabsf(v))); }
 
-template <typename T, int MODE, int NPL>  // NPL: state entries per lane (>= ceil(N / 4))
+// NPL: state entries per lane (>= ceil(N / 4)); CH: tokens staged per round
+template <typename T, int MODE, int NPL, int CH>
 __global__ __launch_bounds__(NT) void decay_scan_kernel(DecayScanArgs a) {
   extern __shared__ float lds[];
+  constexpr int NPAD = NPL * SLICES;
+  constexpr int LROW = SLICES * (NPL + 4);                  // a token's LDS row: the four slices 16 bytes apart in bank
+                                                            // space, so the lanes' four addresses of a read do not collide
+  constexpr int EPT = CH * NPAD / NT;                       // staged (token, channel) entries per thread
+  constexpr int ASZ = MODE == 0 ? CH * LROW : 2 * CH;       // decays per channel, or (decay, step) per token
+  constexpr int BUF = 2 * CH * LROW + ASZ;
+  static_assert(CH * NPAD % NT == 0, "staging split");
   const int N = a.N, P = a.P;
-  const int npad = NPL * SLICES;
-  float* qS = lds;                    // [CH][npad]
-  float* kS = qS + CH * npad;         // [CH][npad]
-  float* aS = kS + CH * npad;         // [CH][npad] (mode 0) or [CH] (mode 1)
-  float* bS = aS + (MODE == 0 ? CH * npad : CH);  // [CH] (mode 1)
   const int h = blockIdx.y, run = blockIdx.z;
   const int s0 = a.cu_q ? a.cu_q[run] : run, s1 = a.cu_q ? a.cu_q[run + 1] : run + 1;
   if (s1 <= s0) return;
@@ -44,6 +47,7 @@ __global__ __launch_bounds__(NT) void decay_scan_kernel(DecayScanArgs a) {
   const int p = blockIdx.x * (PCOLS * (NT / 64)) + wave * PCOLS + pc;
   const bool pin = p < P;
   const int n0 = ns * NPL;
+  const int l0 = ns * (NPL + 4);
   const int grp = h / a.hpg;
   const int pr = a.prev_row[s0];
   const int sv = a.save_slot[s1 - 1];
@@ -63,43 +67,67 @@ __global__ __launch_bounds__(NT) void decay_scan_kernel(DecayScanArgs a) {
   const float skip = a.skip ? a.skip[h] : 0.f;
   const float inv_tau = MODE == 0 ? 1.f / a.tau : 0.f;
   const float rate = MODE == 1 ? expf(a.rate[h]) : 0.f;
-  for (int t0 = s0; t0 < s1; t0 += CH) {
+  // a round's inputs travel global -> registers (issued before the previous round is computed) -> LDS (with the
+  // transcendental part of the decay evaluated once per (token, channel)); two LDS buffers, one barrier per round
+  float rq[EPT], rk[EPT], rz[EPT], vn[CH], rdt = 0.f;
+  auto fetch = [&](int t0) {
     const int nt = min(CH, s1 - t0);
-    __syncthreads();   // the previous round's vectors have been used
-    for (int i = threadIdx.x; i < nt * npad; i += NT) {
-      const int tt = i / npad, n = i - tt * npad;
+#pragma unroll
+    for (int u = 0; u < EPT; ++u) {
+      const int i = threadIdx.x + NT * u;
+      const int tt = i / NPAD, n = i - tt * NPAD;
+      const bool in = tt < nt && n < N;
       const long long r = t0 + tt;
-      float qv = 0.f, kv = 0.f, av = 1.f;
-      if (n < N) {
-        qv = (float)q[r * a.ldq + n] * a.q_scale;
-        kv = (float)k[r * a.ldk + n];
-        if (MODE == 0) {
-          const float z = (float)dz[r * a.ldd + (long long)h * N + n] + a.dbias[(long long)h * N + n];
-          av = expf(-softplus_exact(-z) * inv_tau);   // logsigmoid(z) = -softplus(-z)
-        }
-      }
-      qS[i] = qv;
-      kS[i] = kv;
-      if (MODE == 0) aS[i] = av;
+      rq[u] = in ? (float)q[r * a.ldq + n] : 0.f;
+      rk[u] = in ? (float)k[r * a.ldk + n] : 0.f;
+      if (MODE == 0) rz[u] = in ? (float)dz[r * a.ldd + (long long)h * N + n] + a.dbias[(long long)h * N + n] : 0.f;
     }
-    if (MODE == 1 && threadIdx.x < nt) {
-      const long long r = t0 + threadIdx.x;
-      const float b = softplus_exact((float)dz[r * a.ldd + h] + a.dbias[h]);
-      bS[threadIdx.x] = b;
+    if (MODE == 1 && threadIdx.x < CH)
+      rdt = (int)threadIdx.x < nt ? (float)dz[(long long)(t0 + threadIdx.x) * a.ldd + h] + a.dbias[h] : 0.f;
+#pragma unroll
+    for (int tt = 0; tt < CH; ++tt) vn[tt] = (tt < nt && pin) ? (float)v[(long long)(t0 + tt) * a.ldv] : 0.f;
+  };
+  auto commit = [&](float* buf) {
+    float* qS = buf;
+    float* kS = buf + CH * LROW;
+    float* aS = kS + CH * LROW;
+#pragma unroll
+    for (int u = 0; u < EPT; ++u) {
+      const int i = threadIdx.x + NT * u;
+      const int tt = i / NPAD, n = i - tt * NPAD;
+      const int o = tt * LROW + (n / NPL) * (NPL + 4) + n % NPL;
+      qS[o] = rq[u] * a.q_scale;
+      kS[o] = rk[u];
+      if (MODE == 0) aS[o] = expf(-softplus_exact(-rz[u]) * inv_tau);   // logsigmoid(z) = -softplus(-z); padding: k = q = 0
+    }
+    if (MODE == 1 && threadIdx.x < CH) {
+      const float b = softplus_exact(rdt);
       aS[threadIdx.x] = expf(-rate * b);
+      aS[CH + threadIdx.x] = b;
     }
+  };
+  fetch(s0);
+  int flip = 0;
+  for (int t0 = s0; t0 < s1; t0 += CH, flip ^= 1) {
+    const int nt = min(CH, s1 - t0);
+    float* buf = lds + flip * BUF;
+    commit(buf);
     float vr[CH];
 #pragma unroll
-    for (int tt = 0; tt < CH; ++tt) vr[tt] = (tt < nt && pin) ? (float)v[(long long)(t0 + tt) * a.ldv] : 0.f;
-    __syncthreads();
+    for (int tt = 0; tt < CH; ++tt) vr[tt] = vn[tt];
+    __syncthreads();   // this round's vectors are in LDS; every thread has finished the round before the last (same buffer)
+    if (t0 + CH < s1) fetch(t0 + CH);
+    const float* qS = buf;
+    const float* kS = buf + CH * LROW;
+    const float* aS = kS + CH * LROW;
 #pragma unroll
     for (int tt = 0; tt < CH; ++tt) {
       if (tt < nt) {
-        const float* qr = qS + tt * npad + n0;
-        const float* kr = kS + tt * npad + n0;
+        const float* qr = qS + tt * LROW + l0;
+        const float* kr = kS + tt * LROW + l0;
         float u = vr[tt], o = 0.f;
         if (MODE == 1) {
-          u *= bS[tt];
+          u *= aS[CH + tt];
           const float at = aS[tt];
 #pragma unroll
           for (int i = 0; i < NPL; ++i) {
@@ -107,7 +135,7 @@ __global__ __launch_bounds__(NT) void decay_scan_kernel(DecayScanArgs a) {
             o += S[i] * qr[i];
           }
         } else {
-          const float* ar = aS + tt * npad + n0;
+          const float* ar = aS + tt * LROW + l0;
 #pragma unroll
           for (int i = 0; i < NPL; ++i) {
             S[i] = ar[i] * S[i] + kr[i] * u;
@@ -128,20 +156,23 @@ __global__ __launch_bounds__(NT) void decay_scan_kernel(DecayScanArgs a) {
   }
 }
 
-template <typename T, int MODE>
-void launch_mode(const DecayScanArgs& a, hipStream_t s) {
+template <typename T, int MODE, int NPL, int CH>
+void launch_one(const DecayScanArgs& a, hipStream_t s) {
   const int cols = PCOLS * (NT / 64);
   dim3 grid((a.P + cols - 1) / cols, a.H, a.runs);
+  const int lrow = SLICES * (NPL + 4);
+  const size_t lds = (size_t)2 * (2 * CH * lrow + (MODE == 0 ? CH * lrow : 2 * CH)) * sizeof(float);
+  decay_scan_kernel<T, MODE, NPL, CH><<<grid, NT, lds, s>>>(a);
+}
+
+template <typename T, int MODE>
+void launch_mode(const DecayScanArgs& a, hipStream_t s) {
   const int need = (a.N + SLICES - 1) / SLICES;
-  auto lds = [&](int npl) {
-    const int npad = npl * SLICES;
-    return (size_t)(CH * npad * 2 + (MODE == 0 ? CH * npad : 2 * CH)) * sizeof(float);
-  };
-  if (need <= 4) decay_scan_kernel<T, MODE, 4><<<grid, NT, lds(4), s>>>(a);
-  else if (need <= 8) decay_scan_kernel<T, MODE, 8><<<grid, NT, lds(8), s>>>(a);
-  else if (need <= 16) decay_scan_kernel<T, MODE, 16><<<grid, NT, lds(16), s>>>(a);
-  else if (need <= 32) decay_scan_kernel<T, MODE, 32><<<grid, NT, lds(32), s>>>(a);
-  else decay_scan_kernel<T, MODE, 64><<<grid, NT, lds(64), s>>>(a);   // N <= 256 (checked by the op layer)
+  if (need <= 4) launch_one<T, MODE, 4, 16>(a, s);
+  else if (need <= 8) launch_one<T, MODE, 8, 16>(a, s);
+  else if (need <= 16) launch_one<T, MODE, 16, 16>(a, s);
+  else if (need <= 32) launch_one<T, MODE, 32, 16>(a, s);
+  else launch_one<T, MODE, 64, 8>(a, s);   // N <= 256 (checked by the op layer); half the round keeps LDS under 64 KB
 }
 
 }  // namespace

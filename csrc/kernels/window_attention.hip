@@ -74,8 +74,9 @@ __global__ __launch_bounds__(64 * NW) void window_attn_wave_kernel(WindowAttnArg
   for (int t0 = j0 + 64 * wave; t0 <= p; t0 += 64 * NW) {
     const int j = t0 + lane;
     float s = -INFINITY;
+    long long slot = 0;                       // lanes past the row's position: weight 0 on a finite row (slot 0)
     if (j <= p) {
-      const long long slot = (long long)bt[j / a.BS] * a.BS + j % a.BS;
+      slot = (long long)bt[j / a.BS] * a.BS + j % a.BS;
       s = dot_row<T>(kc + (slot * a.G + g) * a.dk, qs, a.dk);
     }
     const float mt = fmaxf(m, wave_max(s));
@@ -86,15 +87,27 @@ __global__ __launch_bounds__(64 * NW) void window_attn_wave_kernel(WindowAttnArg
 #pragma unroll
     for (int i = 0; i < MAX_VCOLS; ++i) acc[i] *= corr;
     const int nt = min(64, p - t0 + 1);
-    for (int jj = 0; jj < nt; ++jj) {
-      const int jk = t0 + jj;
-      const long long slot = (long long)bt[jk / a.BS] * a.BS + jk % a.BS;
-      const T* vr = vc + (slot * a.G + g) * a.dv;
-      const float pw = __shfl(w, jj, 64);     // (uniform index: a lane read, no LDS)
+    const int vslot = (int)slot;              // (cache rows fit 31 bits: checked by the op layer)
+    // eight value rows in flight per round: their cache rows come lane by lane from the scoring phase (no block-table
+    // walk in this loop), the loads of a round are issued together
+    for (int jj = 0; jj < nt; jj += 8) {
+      float pw[8];
+      const T* vr[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        pw[u] = __shfl(w, jj + u, 64);
+        vr[u] = vc + ((long long)__shfl(vslot, jj + u, 64) * a.G + g) * a.dv;
+      }
 #pragma unroll
       for (int i = 0; i < MAX_VCOLS; ++i) {
         const int c = lane + 64 * i;
-        if (c < a.dv) acc[i] += pw * (float)vr[c];
+        if (c < a.dv) {
+          float vv[8];
+#pragma unroll
+          for (int u = 0; u < 8; ++u) vv[u] = (float)vr[u][c];
+#pragma unroll
+          for (int u = 0; u < 8; ++u) acc[i] += pw[u] * vv[u];
+        }
       }
     }
   }
@@ -195,17 +208,29 @@ __global__ __launch_bounds__(256) void window_attn_tile_kernel(WindowAttnArgs a)
       }
       *reinterpret_cast<uint4*>(Ks + key * KS + 8 * ch) = v;
     }
-    for (int id = threadIdx.x; id < 64 * (DV / 8); id += 256) {
-      const int ch = id / 64, key = id - ch * 64;   // consecutive lanes: consecutive keys of one column group
+    // values transposed: a thread takes 8 columns of two neighbouring keys and stores them as eight 4-byte words (a key
+    // pair per word), consecutive lanes writing consecutive words of a column's row.  (Fetching the next tile into
+    // registers ahead of the products measured slower: the workgroups sharing a CU already cover the load latency.)
+    for (int id = threadIdx.x; id < 32 * (DV / 8); id += 256) {
+      const int ch = id / 32, key = 2 * (id - ch * 32);
+      Pack8 va, vb;
+      va.u = vb.u = make_uint4(0, 0, 0, 0);
       const int kp = kt + key;
-      Pack8 v;
-      v.u = make_uint4(0, 0, 0, 0);
       if (kp <= p_last) {
         const long long slot = (long long)bt[kp / a.BS] * a.BS + kp % a.BS;
-        v.u = *reinterpret_cast<const uint4*>(vc + (slot * a.G + g) * DV + 8 * ch);
+        va.u = *reinterpret_cast<const uint4*>(vc + (slot * a.G + g) * DV + 8 * ch);
+      }
+      if (kp + 1 <= p_last) {
+        const long long slot = (long long)bt[(kp + 1) / a.BS] * a.BS + (kp + 1) % a.BS;
+        vb.u = *reinterpret_cast<const uint4*>(vc + (slot * a.G + g) * DV + 8 * ch);
       }
 #pragma unroll
-      for (int i = 0; i < 8; ++i) Vt[(8 * ch + i) * VS + key] = v.h[i];
+      for (int m2 = 0; m2 < 4; ++m2) {
+        const unsigned int wa = va.w[m2], wb = vb.w[m2];
+        unsigned int* dst = reinterpret_cast<unsigned int*>(Vt + (8 * ch + 2 * m2) * VS + key);
+        dst[0] = (wa & 0xffffu) | (wb << 16);
+        dst[VS / 2] = (wa >> 16) | (wb & 0xffff0000u);
+      }
     }
     __syncthreads();
     // scores: sc[s][e] = q_j . k_(kt + 16 s + 4 hq + e)
