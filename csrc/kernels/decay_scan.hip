@@ -14,8 +14,8 @@
 // lanes are 16 columns x 4 slices of the key channels, so a lane keeps N / 4 state entries of one column in
 // registers and a token's output is a 4-lane sum (two cross-lane adds).  The per-token vectors that all columns
 // share (q, k, the decays) are staged through LDS for CH tokens at a time by the whole workgroup, with the
-// transcendental part of the decay evaluated once per (token, channel) there; the next round's global loads are in
-// flight while the current round is computed (two LDS buffers, one barrier per round).
+// transcendental part of the decay evaluated once per (token, channel) there; the next batch's global loads are in
+// flight while the current batch is computed (two LDS buffers, one barrier per batch).
 #include "common.h"
 #include "hybrid_launchers.h"
 
@@ -27,7 +27,7 @@ constexpr int SLICES = 4;   // key-channel slices per column (lanes)
 
 SYM_DEV float softplus_exact(float v) { return fmaxf(v, 0.f) + log1pf(expf(-fabsf(v))); }
 
-// NPL: state entries per lane (>= ceil(N / 4)); CH: tokens staged per round
+// NPL: state entries per lane (>= ceil(N / 4)); CH: tokens staged per batch
 template <typename T, int MODE, int NPL, int CH>
 __global__ __launch_bounds__(NT) void decay_scan_kernel(DecayScanArgs a) {
   extern __shared__ float lds[];
@@ -67,8 +67,8 @@ __global__ __launch_bounds__(NT) void decay_scan_kernel(DecayScanArgs a) {
   const float skip = a.skip ? a.skip[h] : 0.f;
   const float inv_tau = MODE == 0 ? 1.f / a.tau : 0.f;
   const float rate = MODE == 1 ? expf(a.rate[h]) : 0.f;
-  // a round's inputs travel global -> registers (issued before the previous round is computed) -> LDS (with the
-  // transcendental part of the decay evaluated once per (token, channel)); two LDS buffers, one barrier per round
+  // a batch's inputs travel global -> registers (issued before the previous batch is computed) -> LDS (with the
+  // transcendental part of the decay evaluated once per (token, channel)); two LDS buffers, one barrier per batch
   float rq[EPT], rk[EPT], rz[EPT], vn[CH], rdt = 0.f;
   auto fetch = [&](int t0) {
     const int nt = min(CH, s1 - t0);
@@ -115,7 +115,7 @@ __global__ __launch_bounds__(NT) void decay_scan_kernel(DecayScanArgs a) {
     float vr[CH];
 #pragma unroll
     for (int tt = 0; tt < CH; ++tt) vr[tt] = vn[tt];
-    __syncthreads();   // this round's vectors are in LDS; every thread has finished the round before the last (same buffer)
+    __syncthreads();   // this batch's vectors are in LDS; every thread has finished the batch before the last (same buffer)
     if (t0 + CH < s1) fetch(t0 + CH);
     const float* qS = buf;
     const float* kS = buf + CH * LROW;
@@ -172,7 +172,7 @@ void launch_mode(const DecayScanArgs& a, hipStream_t s) {
   else if (need <= 8) launch_one<T, MODE, 8, 16>(a, s);
   else if (need <= 16) launch_one<T, MODE, 16, 16>(a, s);
   else if (need <= 32) launch_one<T, MODE, 32, 16>(a, s);
-  else launch_one<T, MODE, 64, 8>(a, s);   // N <= 256 (checked by the op layer); half the round keeps LDS under 64 KB
+  else launch_one<T, MODE, 64, 8>(a, s);   // N <= 256 (checked by the op layer); half the batch keeps LDS under 64 KB
 }
 
 }  // namespace

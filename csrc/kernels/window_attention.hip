@@ -88,8 +88,8 @@ __global__ __launch_bounds__(64 * NW) void window_attn_wave_kernel(WindowAttnArg
     for (int i = 0; i < MAX_VCOLS; ++i) acc[i] *= corr;
     const int nt = min(64, p - t0 + 1);
     const int vslot = (int)slot;              // (cache rows fit 31 bits: checked by the op layer)
-    // eight value rows in flight per round: their cache rows come lane by lane from the scoring phase (no block-table
-    // walk in this loop), the loads of a round are issued together
+    // eight value rows in flight per batch: their cache rows come lane by lane from the scoring phase (no block-table
+    // walk in this loop), the loads of a batch are issued together
     for (int jj = 0; jj < nt; jj += 8) {
       float pw[8];
       const T* vr[8];
@@ -161,17 +161,17 @@ void launch_wave(const WindowAttnArgs& a, hipStream_t s) {
 // subtile: the row statistics are two cross-lane steps), the weights go back into the MFMA as bf16 against the
 // transposed values with the keys in the order the score fragments already have.  Statistics, masks and the running
 // rescale are fp32.
-template <int DK, int DV>
-__global__ __launch_bounds__(256) void window_attn_tile_kernel(WindowAttnArgs a) {
-  constexpr int KD = DK / 32, VD = DV / 16, KS = DK + 8, VS = 64 + 8;
+template <int DK, int DV, int RW>   // RW waves: 16 RW query rows per workgroup (RW = 8: the even tiles of the list, two each)
+__global__ __launch_bounds__(64 * RW) void window_attn_tile_kernel(WindowAttnArgs a) {
+  constexpr int KD = DK / 32, VD = DV / 16, KS = DK + 8, VS = 64 + 8, NTH = 64 * RW;
   extern __shared__ __attribute__((aligned(16))) char smem[];
   bf16* Ks = reinterpret_cast<bf16*>(smem);   // [64][KS]
   bf16* Vt = Ks + 64 * KS;                    // [DV][VS]
   const int tile = blockIdx.x, h = blockIdx.y;
   const int seq = a.tiles[2 * tile], row0 = a.tiles[2 * tile + 1];
   const int r_hi = a.cu_q[seq + 1], first = a.cu_q[seq] + row0;
-  if (first >= r_hi) return;                  // padding tile (the whole workgroup)
-  const int nrows = min(64, r_hi - first);
+  if (first >= r_hi || (RW == 8 && (row0 & 64))) return;   // padding tile / the second half of a pair (whole workgroup)
+  const int nrows = min(16 * RW, r_hi - first);
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int j = lane & 15, hq = lane >> 4;
   const int g = h / (a.H / a.G);
@@ -198,7 +198,7 @@ __global__ __launch_bounds__(256) void window_attn_tile_kernel(WindowAttnArgs a)
   const int k_lo = max(0, p_first - a.window + 1);
   for (int kt = k_lo & ~63; kt <= p_last; kt += 64) {
     __syncthreads();                          // every wave is done with the previous tile
-    for (int id = threadIdx.x; id < 64 * (DK / 8); id += 256) {
+    for (int id = threadIdx.x; id < 64 * (DK / 8); id += NTH) {
       const int key = id / (DK / 8), ch = id - key * (DK / 8);
       const int kp = kt + key;
       uint4 v = make_uint4(0, 0, 0, 0);
@@ -211,7 +211,7 @@ __global__ __launch_bounds__(256) void window_attn_tile_kernel(WindowAttnArgs a)
     // values transposed: a thread takes 8 columns of two neighbouring keys and stores them as eight 4-byte words (a key
     // pair per word), consecutive lanes writing consecutive words of a column's row.  (Fetching the next tile into
     // registers ahead of the products measured slower: the workgroups sharing a CU already cover the load latency.)
-    for (int id = threadIdx.x; id < 32 * (DV / 8); id += 256) {
+    for (int id = threadIdx.x; id < 32 * (DV / 8); id += NTH) {
       const int ch = id / 32, key = 2 * (id - ch * 32);
       Pack8 va, vb;
       va.u = vb.u = make_uint4(0, 0, 0, 0);
@@ -309,22 +309,24 @@ __global__ __launch_bounds__(256) void window_attn_tile_kernel(WindowAttnArgs a)
 }
 
 template <int D>
-void launch_tile(const WindowAttnArgs& a, hipStream_t s) {
+void launch_tile(const WindowAttnArgs& a, int rw, hipStream_t s) {
   dim3 grid(a.ntiles, a.H);
   const size_t lds = (size_t)(64 * (D + 8) + D * (64 + 8)) * sizeof(bf16);
-  window_attn_tile_kernel<D, D><<<grid, 256, lds, s>>>(a);
+  if (rw == 8) window_attn_tile_kernel<D, D, 8><<<grid, 512, lds, s>>>(a);
+  else window_attn_tile_kernel<D, D, 4><<<grid, 256, lds, s>>>(a);
 }
 
 }  // namespace
 
 int launch_window_attn(const WindowAttnArgs& a, int f32, int impl, hipStream_t s) {
   if (a.T <= 0) return 0;
-  if (impl == 1 && !f32 && a.tiles && a.cu_q && a.ntiles > 0 && a.dk == a.dv && a.ntiles <= 65535 * 16) {
+  if (impl >= 1 && !f32 && a.tiles && a.cu_q && a.ntiles > 0 && a.dk == a.dv && a.ntiles <= 65535 * 16) {
+    const int rw = impl == 2 ? 8 : 4;
     switch (a.dk) {
-      case 32: launch_tile<32>(a, s); return 1;
-      case 64: launch_tile<64>(a, s); return 1;
-      case 96: launch_tile<96>(a, s); return 1;
-      case 128: launch_tile<128>(a, s); return 1;
+      case 32: launch_tile<32>(a, rw, s); return 1;
+      case 64: launch_tile<64>(a, rw, s); return 1;
+      case 96: launch_tile<96>(a, rw, s); return 1;
+      case 128: launch_tile<128>(a, rw, s); return 1;
       default: break;
     }
   }
