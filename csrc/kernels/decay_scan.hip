@@ -22,15 +22,16 @@
 namespace {
 
 constexpr int NT = 256;
-constexpr int PCOLS = 16;   // value columns per wave
-constexpr int SLICES = 4;   // key-channel slices per column (lanes)
+// A wave's lanes are PCOLS value columns x SLICES slices of the key channels (PCOLS * SLICES = 64): 16 x 4, or 8 x 8
+// when heads x columns x sequences would leave SIMDs with a single wave (more, shorter waves hide each other's latency).
 
 SYM_DEV float softplus_exact(float v) { return fmaxf(v, 0.f) + log1pf(expf(-fabsf(v))); }
 
-// NPL: state entries per lane (>= ceil(N / 4)); CH: tokens staged per batch
-template <typename T, int MODE, int NPL, int CH>
+// NPL: state entries per lane (>= ceil(N / SLICES)); CH: tokens staged per batch
+template <typename T, int MODE, int NPL, int CH, int SLICES>
 __global__ __launch_bounds__(NT) void decay_scan_kernel(DecayScanArgs a) {
   extern __shared__ float lds[];
+  constexpr int PCOLS = 64 / SLICES;
   constexpr int NPAD = NPL * SLICES;
   constexpr int LROW = SLICES * (NPL + 4);                  // a token's LDS row: the four slices 16 bytes apart in bank
                                                             // space, so the lanes' four addresses of a read do not collide
@@ -43,7 +44,7 @@ __global__ __launch_bounds__(NT) void decay_scan_kernel(DecayScanArgs a) {
   const int s0 = a.cu_q ? a.cu_q[run] : run, s1 = a.cu_q ? a.cu_q[run + 1] : run + 1;
   if (s1 <= s0) return;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int pc = lane & (PCOLS - 1), ns = lane >> 4;
+  const int pc = lane & (PCOLS - 1), ns = lane / PCOLS;
   const int p = blockIdx.x * (PCOLS * (NT / 64)) + wave * PCOLS + pc;
   const bool pin = p < P;
   const int n0 = ns * NPL;
@@ -120,33 +121,54 @@ __global__ __launch_bounds__(NT) void decay_scan_kernel(DecayScanArgs a) {
     const float* qS = buf;
     const float* kS = buf + CH * LROW;
     const float* aS = kS + CH * LROW;
+    float po[CH];
 #pragma unroll
     for (int tt = 0; tt < CH; ++tt) {
+      po[tt] = 0.f;
       if (tt < nt) {
         const float* qr = qS + tt * LROW + l0;
         const float* kr = kS + tt * LROW + l0;
-        float u = vr[tt], o = 0.f;
+        float u = vr[tt], o0 = 0.f, o1 = 0.f, o2 = 0.f, o3 = 0.f;
+        // 16-byte LDS reads (rows, slices and buffers all start at multiples of four floats)
+        const float4* q4 = reinterpret_cast<const float4*>(qr);
+        const float4* k4 = reinterpret_cast<const float4*>(kr);
         if (MODE == 1) {
           u *= aS[CH + tt];
           const float at = aS[tt];
 #pragma unroll
-          for (int i = 0; i < NPL; ++i) {
-            S[i] = at * S[i] + kr[i] * u;
-            o += S[i] * qr[i];
+          for (int i = 0; i < NPL / 4; ++i) {
+            const float4 kv = k4[i], qv = q4[i];
+            S[4 * i + 0] = at * S[4 * i + 0] + kv.x * u;
+            S[4 * i + 1] = at * S[4 * i + 1] + kv.y * u;
+            S[4 * i + 2] = at * S[4 * i + 2] + kv.z * u;
+            S[4 * i + 3] = at * S[4 * i + 3] + kv.w * u;
+            o0 += S[4 * i + 0] * qv.x, o1 += S[4 * i + 1] * qv.y, o2 += S[4 * i + 2] * qv.z, o3 += S[4 * i + 3] * qv.w;
           }
         } else {
-          const float* ar = aS + tt * LROW + l0;
+          const float4* a4 = reinterpret_cast<const float4*>(aS + tt * LROW + l0);
 #pragma unroll
-          for (int i = 0; i < NPL; ++i) {
-            S[i] = ar[i] * S[i] + kr[i] * u;
-            o += S[i] * qr[i];
+          for (int i = 0; i < NPL / 4; ++i) {
+            const float4 kv = k4[i], qv = q4[i], av = a4[i];
+            S[4 * i + 0] = av.x * S[4 * i + 0] + kv.x * u;
+            S[4 * i + 1] = av.y * S[4 * i + 1] + kv.y * u;
+            S[4 * i + 2] = av.z * S[4 * i + 2] + kv.z * u;
+            S[4 * i + 3] = av.w * S[4 * i + 3] + kv.w * u;
+            o0 += S[4 * i + 0] * qv.x, o1 += S[4 * i + 1] * qv.y, o2 += S[4 * i + 2] * qv.z, o3 += S[4 * i + 3] * qv.w;
           }
         }
-        o += __shfl_xor(o, 16, 64);
-        o += __shfl_xor(o, 32, 64);
-        if (ns == 0 && pin) a.out[((long long)(t0 + tt) * a.H + h) * P + p] = o + skip * vr[tt];
+        po[tt] = (o0 + o1) + (o2 + o3);
       }
     }
+    // the slices' partial sums of the whole batch meet in one go: the tokens' cross-lane adds are independent of one
+    // another, so their latencies overlap (done per token they sat on the serial path)
+#pragma unroll
+    for (int sh = PCOLS; sh < 64; sh <<= 1)
+#pragma unroll
+      for (int tt = 0; tt < CH; ++tt) po[tt] += __shfl_xor(po[tt], sh, 64);
+    if (ns == 0 && pin)
+#pragma unroll
+      for (int tt = 0; tt < CH; ++tt)
+        if (tt < nt) a.out[((long long)(t0 + tt) * a.H + h) * P + p] = po[tt] + skip * vr[tt];
   }
   if (sv >= 0 && pin) {
     float* st = a.state + (long long)sv * a.state_stride + (long long)h * N * P + p;
@@ -156,23 +178,32 @@ __global__ __launch_bounds__(NT) void decay_scan_kernel(DecayScanArgs a) {
   }
 }
 
-template <typename T, int MODE, int NPL, int CH>
+template <typename T, int MODE, int NPL, int CH, int SLICES>
 void launch_one(const DecayScanArgs& a, hipStream_t s) {
-  const int cols = PCOLS * (NT / 64);
+  const int cols = (64 / SLICES) * (NT / 64);
   dim3 grid((a.P + cols - 1) / cols, a.H, a.runs);
   const int lrow = SLICES * (NPL + 4);
   const size_t lds = (size_t)2 * (2 * CH * lrow + (MODE == 0 ? CH * lrow : 2 * CH)) * sizeof(float);
-  decay_scan_kernel<T, MODE, NPL, CH><<<grid, NT, lds, s>>>(a);
+  decay_scan_kernel<T, MODE, NPL, CH, SLICES><<<grid, NT, lds, s>>>(a);
 }
 
 template <typename T, int MODE>
 void launch_mode(const DecayScanArgs& a, hipStream_t s) {
-  const int need = (a.N + SLICES - 1) / SLICES;
-  if (need <= 4) launch_one<T, MODE, 4, 16>(a, s);
-  else if (need <= 8) launch_one<T, MODE, 8, 16>(a, s);
-  else if (need <= 16) launch_one<T, MODE, 16, 16>(a, s);
-  else if (need <= 32) launch_one<T, MODE, 32, 16>(a, s);
-  else launch_one<T, MODE, 64, 8>(a, s);   // N <= 256 (checked by the op layer); half the batch keeps LDS under 64 KB
+  // waves with 16 columns each; under two per SIMD (1024 SIMDs) and enough key channels: 8 columns x 8 slices
+  const long long waves16 = (long long)a.runs * a.H * ((a.P + 15) / 16);
+  if (waves16 < 2048 && a.N >= 64 && a.T > a.runs) {
+    const int need = (a.N + 7) / 8;
+    if (need <= 8) launch_one<T, MODE, 8, 16, 8>(a, s);
+    else if (need <= 16) launch_one<T, MODE, 16, 16, 8>(a, s);
+    else launch_one<T, MODE, 32, 8, 8>(a, s);      // N <= 256 (checked by the op layer)
+    return;
+  }
+  const int need = (a.N + 3) / 4;
+  if (need <= 4) launch_one<T, MODE, 4, 16, 4>(a, s);
+  else if (need <= 8) launch_one<T, MODE, 8, 16, 4>(a, s);
+  else if (need <= 16) launch_one<T, MODE, 16, 16, 4>(a, s);
+  else if (need <= 32) launch_one<T, MODE, 32, 16, 4>(a, s);
+  else launch_one<T, MODE, 64, 8, 4>(a, s);   // N <= 256; half the batch keeps LDS under 64 KB
 }
 
 }  // namespace
