@@ -89,6 +89,7 @@ struct WindowAttnArgs {
   long long ldg;
   void* out;            // [T][H][dv]
   int T, H, G, dk, dv, BS, max_blocks, window;
+  int bs_shift;         // log2(BS), or -1 if BS is no power of two (set by the launcher)
   float scale;
   // packed prompt form for the tiled kernel: 64-row query tiles (sequence, first row within the run)
   const int* tiles;

@@ -16,6 +16,11 @@ namespace {
 
 constexpr int MAX_VCOLS = 8;  // value columns per lane: dv <= 512
 
+// cache row of position kp of a sequence (block table bt): a shift and a mask for power-of-two blocks
+SYM_DEV long long cache_row(const int* __restrict__ bt, int kp, int BS, int shift) {
+  return shift >= 0 ? ((long long)bt[kp >> shift] << shift) + (kp & (BS - 1)) : (long long)bt[kp / BS] * BS + kp % BS;
+}
+
 template <typename T>
 SYM_DEV float dot_row(const T* __restrict__ k, const float* __restrict__ q, int dk);
 
@@ -76,7 +81,7 @@ __global__ __launch_bounds__(64 * NW) void window_attn_wave_kernel(WindowAttnArg
     float s = -INFINITY;
     long long slot = 0;                       // lanes past the row's position: weight 0 on a finite row (slot 0)
     if (j <= p) {
-      slot = (long long)bt[j / a.BS] * a.BS + j % a.BS;
+      slot = cache_row(bt, j, a.BS, a.bs_shift);
       s = dot_row<T>(kc + (slot * a.G + g) * a.dk, qs, a.dk);
     }
     const float mt = fmaxf(m, wave_max(s));
@@ -195,6 +200,7 @@ __global__ __launch_bounds__(64 * RW) void window_attn_tile_kernel(WindowAttnArg
 #pragma unroll
   for (int i = 0; i < VD; ++i) o[i] = f32x4{0.f, 0.f, 0.f, 0.f};
   float m = -INFINITY, l = 0.f;
+  const float sl2 = a.scale * 1.44269504088896341f;
   const int k_lo = max(0, p_first - a.window + 1);
   for (int kt = k_lo & ~63; kt <= p_last; kt += 64) {
     __syncthreads();                          // every wave is done with the previous tile
@@ -203,7 +209,7 @@ __global__ __launch_bounds__(64 * RW) void window_attn_tile_kernel(WindowAttnArg
       const int kp = kt + key;
       uint4 v = make_uint4(0, 0, 0, 0);
       if (kp <= p_last) {
-        const long long slot = (long long)bt[kp / a.BS] * a.BS + kp % a.BS;
+        const long long slot = cache_row(bt, kp, a.BS, a.bs_shift);
         v = *reinterpret_cast<const uint4*>(kc + (slot * a.G + g) * DK + 8 * ch);
       }
       *reinterpret_cast<uint4*>(Ks + key * KS + 8 * ch) = v;
@@ -217,11 +223,11 @@ __global__ __launch_bounds__(64 * RW) void window_attn_tile_kernel(WindowAttnArg
       va.u = vb.u = make_uint4(0, 0, 0, 0);
       const int kp = kt + key;
       if (kp <= p_last) {
-        const long long slot = (long long)bt[kp / a.BS] * a.BS + kp % a.BS;
+        const long long slot = cache_row(bt, kp, a.BS, a.bs_shift);
         va.u = *reinterpret_cast<const uint4*>(vc + (slot * a.G + g) * DV + 8 * ch);
       }
       if (kp + 1 <= p_last) {
-        const long long slot = (long long)bt[(kp + 1) / a.BS] * a.BS + (kp + 1) % a.BS;
+        const long long slot = cache_row(bt, kp + 1, a.BS, a.bs_shift);
         vb.u = *reinterpret_cast<const uint4*>(vc + (slot * a.G + g) * DV + 8 * ch);
       }
 #pragma unroll
@@ -233,7 +239,10 @@ __global__ __launch_bounds__(64 * RW) void window_attn_tile_kernel(WindowAttnArg
       }
     }
     __syncthreads();
-    // scores: sc[s][e] = q_j . k_(kt + 16 s + 4 hq + e)
+    // scores in units of log2(e): sc[s][e] = scale * log2(e) * q_j . k_(kt + 16 s + 4 hq + e).  A key tile that every
+    // row of the wave sees completely (the usual case away from the diagonal and the window's far edge) skips the masks.
+    const int wq_lo = p_first + 16 * wave, wq_hi = wq_lo + 15;
+    const bool interior = 16 * wave + 15 < nrows && kt + 63 <= wq_lo && kt > wq_hi - a.window;
     float pv[4][4];
     float mx = -INFINITY;
 #pragma unroll
@@ -245,12 +254,20 @@ __global__ __launch_bounds__(64 * RW) void window_attn_tile_kernel(WindowAttnArg
         kf.u = *reinterpret_cast<const uint4*>(Ks + (16 * s4 + j) * KS + 32 * kk + 8 * hq);
         acc = mfma16(kf.v, qf[kk].v, acc);
       }
+      if (interior) {
 #pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        const int kp = kt + 16 * s4 + 4 * hq + e;
-        const bool vis = rv && kp <= qp && kp > qp - a.window;
-        pv[s4][e] = vis ? acc[e] * a.scale : -INFINITY;
-        mx = fmaxf(mx, pv[s4][e]);
+        for (int e = 0; e < 4; ++e) {
+          pv[s4][e] = acc[e] * sl2;
+          mx = fmaxf(mx, pv[s4][e]);
+        }
+      } else {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const int kp = kt + 16 * s4 + 4 * hq + e;
+          const bool vis = rv && kp <= qp && kp > qp - a.window;
+          pv[s4][e] = vis ? acc[e] * sl2 : -INFINITY;
+          mx = fmaxf(mx, pv[s4][e]);
+        }
       }
     }
     mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
@@ -262,16 +279,19 @@ __global__ __launch_bounds__(64 * RW) void window_attn_tile_kernel(WindowAttnArg
     for (int s4 = 0; s4 < 4; ++s4)
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
-        pv[s4][e] = __expf(pv[s4][e] - mref);
+        pv[s4][e] = exp2f(pv[s4][e] - mref);
         sum += pv[s4][e];
       }
     sum += __shfl_xor(sum, 16, 64);
     sum += __shfl_xor(sum, 32, 64);
-    const float corr = __expf(m - mref);
-    l = l * corr + sum;
-    m = mt;
+    if (__any(mt > m)) {                             // some row's running max moved: rescale (else every factor is 1)
+      const float corr = exp2f(m - mref);
+      l *= corr;
 #pragma unroll
-    for (int i = 0; i < VD; ++i) o[i] *= corr;
+      for (int i = 0; i < VD; ++i) o[i] *= corr;
+    }
+    l += sum;
+    m = mt;
     // weighted values: key slots of lane group hq in a 32-key chunk c2 are keys 32 c2 + 4 hq + (0..3) and + 16
 #pragma unroll
     for (int c2 = 0; c2 < 2; ++c2) {
@@ -318,8 +338,12 @@ void launch_tile(const WindowAttnArgs& a, int rw, hipStream_t s) {
 
 }  // namespace
 
-int launch_window_attn(const WindowAttnArgs& a, int f32, int impl, hipStream_t s) {
-  if (a.T <= 0) return 0;
+int launch_window_attn(const WindowAttnArgs& args, int f32, int impl, hipStream_t s) {
+  if (args.T <= 0) return 0;
+  WindowAttnArgs a = args;
+  a.bs_shift = -1;
+  for (int b = 0; b < 31; ++b)
+    if (a.BS == 1 << b) a.bs_shift = b;
   if (impl >= 1 && !f32 && a.tiles && a.cu_q && a.ntiles > 0 && a.dk == a.dv && a.ntiles <= 65535 * 16) {
     const int rw = impl == 2 ? 8 : 4;
     switch (a.dk) {
