@@ -28,46 +28,46 @@ SYM_DEV float ldf(const void* p, int f32, long long i) {
 SYM_DEV float sigmoidf(float v) { return 1.f / (1.f + expf(-v)); }
 SYM_DEV float silu_exact(float v) { return v / (1.f + expf(-v)); }
 
-template <typename T>
-__global__ __launch_bounds__(NT) void embed_norm_kernel(const int* __restrict__ ids, const int* __restrict__ src,
+template <typename T, int BT>
+__global__ __launch_bounds__(BT) void embed_norm_kernel(const int* __restrict__ ids, const int* __restrict__ src,
                                                         const int* __restrict__ prev, const T* __restrict__ table,
                                                         const float* __restrict__ w, float eps, float offset,
                                                         float* __restrict__ x, int d) {
-  __shared__ float scratch[NT / 64];
+  __shared__ float scratch[BT / 64];
   const int row = blockIdx.x;
   const int sr = src ? src[row] : -1;
   const long long tok = sr >= 0 ? prev[sr] : ids[row];
   const T* t = table + tok * d;
   float sq = 0.f;
-  for (int c = threadIdx.x; c < d; c += NT) {
+  for (int c = threadIdx.x; c < d; c += BT) {
     const float v = (float)t[c];
     sq += v * v;
   }
-  const float r = 1.f / sqrtf(block_sum<NT>(sq, scratch) / (float)d + eps);
-  for (int c = threadIdx.x; c < d; c += NT) x[(long long)row * d + c] = (float)t[c] * r * (offset + w[c]);
+  const float r = 1.f / sqrtf(block_sum<BT>(sq, scratch) / (float)d + eps);
+  for (int c = threadIdx.x; c < d; c += BT) x[(long long)row * d + c] = (float)t[c] * r * (offset + w[c]);
 }
 
-template <typename T>
-__global__ __launch_bounds__(NT) void rms_norm_rows_kernel(const float* __restrict__ x, const long long* __restrict__ rows,
+template <typename T, int BT>
+__global__ __launch_bounds__(BT) void rms_norm_rows_kernel(const float* __restrict__ x, const long long* __restrict__ rows,
                                                            const float* __restrict__ w, float eps, float offset,
                                                            T* __restrict__ out, int d) {
-  __shared__ float scratch[NT / 64];
+  __shared__ float scratch[BT / 64];
   const int i = blockIdx.x;
   const float* xr = x + (rows ? rows[i] : (long long)i) * d;
   float sq = 0.f;
-  for (int c = threadIdx.x; c < d; c += NT) sq += xr[c] * xr[c];
-  const float r = 1.f / sqrtf(block_sum<NT>(sq, scratch) / (float)d + eps);
-  for (int c = threadIdx.x; c < d; c += NT) out[(long long)i * d + c] = (T)(xr[c] * r * (offset + w[c]));
+  for (int c = threadIdx.x; c < d; c += BT) sq += xr[c] * xr[c];
+  const float r = 1.f / sqrtf(block_sum<BT>(sq, scratch) / (float)d + eps);
+  for (int c = threadIdx.x; c < d; c += BT) out[(long long)i * d + c] = (T)(xr[c] * r * (offset + w[c]));
 }
 
-template <typename T>
-__global__ __launch_bounds__(NT) void residual_mix_norm_kernel(ResidualMixArgs a) {
-  __shared__ float scratch[NT / 64];
+template <typename T, int BT>
+__global__ __launch_bounds__(BT) void residual_mix_norm_kernel(ResidualMixArgs a) {
+  __shared__ float scratch[BT / 64];
   const int row = blockIdx.x, d = a.d;
   float* xr = a.x + (long long)row * d;
   const long long o = (long long)row * d;
   float sq = 0.f;
-  for (int c = threadIdx.x; c < d; c += NT) {
+  for (int c = threadIdx.x; c < d; c += BT) {
     float s = ldf(a.a, a.a_f32, o + c);
     if (a.bias_a) s += a.bias_a[c];
     s *= a.sa;
@@ -78,14 +78,14 @@ __global__ __launch_bounds__(NT) void residual_mix_norm_kernel(ResidualMixArgs a
     sq += xn * xn;
   }
   if (!a.out) return;
-  const float r = 1.f / sqrtf(block_sum<NT>(sq, scratch) / (float)d + a.eps);
+  const float r = 1.f / sqrtf(block_sum<BT>(sq, scratch) / (float)d + a.eps);
   T* out = reinterpret_cast<T*>(a.out) + o;
   // (each thread re-reads the columns it wrote itself)
-  for (int c = threadIdx.x; c < d; c += NT) out[c] = (T)(xr[c] * r * (a.offset + a.w[c]));
+  for (int c = threadIdx.x; c < d; c += BT) out[c] = (T)(xr[c] * r * (a.offset + a.w[c]));
 }
 
-template <typename T>
-__global__ __launch_bounds__(NT) void qkv_rope_cache_kernel(QkvRopeArgs a) {
+template <typename T, int BT>
+__global__ __launch_bounds__(BT) void qkv_rope_cache_kernel(QkvRopeArgs a) {
   const int row = blockIdx.x;
   const T* z = reinterpret_cast<const T*>(a.z) + (long long)row * a.ldz;
   const int nq = a.H * a.dk, nk = a.G * a.dk, nv = a.G * a.dv;
@@ -95,7 +95,7 @@ __global__ __launch_bounds__(NT) void qkv_rope_cache_kernel(QkvRopeArgs a) {
   T* qo = reinterpret_cast<T*>(a.q_out) + (long long)row * nq;
   T* kc = slot >= 0 ? reinterpret_cast<T*>(a.k_cache) + (long long)slot * nk : nullptr;
   T* vc = slot >= 0 ? reinterpret_cast<T*>(a.v_cache) + (long long)slot * nv : nullptr;
-  for (int i = threadIdx.x; i < nq + nk; i += NT) {
+  for (int i = threadIdx.x; i < nq + nk; i += BT) {
     const int e = i < nq ? i % a.dk : (i - nq) % a.dk;   // entry within its head
     float v = (float)z[i] + a.bias[i];
     if (e < rot) {
@@ -108,7 +108,7 @@ __global__ __launch_bounds__(NT) void qkv_rope_cache_kernel(QkvRopeArgs a) {
     else if (kc) kc[i - nq] = (T)v;
   }
   if (vc)
-    for (int i = threadIdx.x; i < nv; i += NT) vc[i] = (T)((float)z[nq + nk + i] + a.bias[nq + nk + i]);
+    for (int i = threadIdx.x; i < nv; i += BT) vc[i] = (T)((float)z[nq + nk + i] + a.bias[nq + nk + i]);
 }
 
 // grid (T, C / group); BT threads over the group's columns
@@ -292,6 +292,9 @@ int ew_grid(long long n) {
 
 }  // namespace
 
+// rows of a decode step: 1024 threads per row make a wide row one or two passes deep instead of eight
+static inline bool wide_rows(int rows, int width) { return rows <= 512 && width >= 1024; }
+
 #define DISPATCH_T(f32, ...)            \
   if (f32) {                            \
     using T = float;                    \
@@ -304,23 +307,39 @@ int ew_grid(long long n) {
 void launch_embed_norm(const int* ids, const int* src, const int* prev, const void* table, const float* w, float eps,
                        float offset, float* x, int T_, int d, int f32, hipStream_t s) {
   if (T_ <= 0) return;
-  DISPATCH_T(f32, embed_norm_kernel<T><<<T_, NT, 0, s>>>(ids, src, prev, (const T*)table, w, eps, offset, x, d);)
+  if (wide_rows(T_, d)) {
+    DISPATCH_T(f32, (embed_norm_kernel<T, 1024><<<T_, 1024, 0, s>>>(ids, src, prev, (const T*)table, w, eps, offset, x, d));)
+  } else {
+    DISPATCH_T(f32, (embed_norm_kernel<T, NT><<<T_, NT, 0, s>>>(ids, src, prev, (const T*)table, w, eps, offset, x, d));)
+  }
 }
 
 void launch_rms_norm_rows(const float* x, const long long* rows, const float* w, float eps, float offset, void* out,
                           int n, int d, int f32, hipStream_t s) {
   if (n <= 0) return;
-  DISPATCH_T(f32, rms_norm_rows_kernel<T><<<n, NT, 0, s>>>(x, rows, w, eps, offset, (T*)out, d);)
+  if (wide_rows(n, d)) {
+    DISPATCH_T(f32, (rms_norm_rows_kernel<T, 1024><<<n, 1024, 0, s>>>(x, rows, w, eps, offset, (T*)out, d));)
+  } else {
+    DISPATCH_T(f32, (rms_norm_rows_kernel<T, NT><<<n, NT, 0, s>>>(x, rows, w, eps, offset, (T*)out, d));)
+  }
 }
 
 void launch_residual_mix_norm(const ResidualMixArgs& a, int f32, hipStream_t s) {
   if (a.T <= 0) return;
-  DISPATCH_T(f32, residual_mix_norm_kernel<T><<<a.T, NT, 0, s>>>(a);)
+  if (wide_rows(a.T, a.d)) {
+    DISPATCH_T(f32, (residual_mix_norm_kernel<T, 1024><<<a.T, 1024, 0, s>>>(a));)
+  } else {
+    DISPATCH_T(f32, (residual_mix_norm_kernel<T, NT><<<a.T, NT, 0, s>>>(a));)
+  }
 }
 
 void launch_qkv_rope_cache(const QkvRopeArgs& a, int T_, int f32, hipStream_t s) {
   if (T_ <= 0) return;
-  DISPATCH_T(f32, qkv_rope_cache_kernel<T><<<T_, NT, 0, s>>>(a);)
+  if (wide_rows(T_, a.H * a.dk)) {
+    DISPATCH_T(f32, (qkv_rope_cache_kernel<T, 1024><<<T_, 1024, 0, s>>>(a));)
+  } else {
+    DISPATCH_T(f32, (qkv_rope_cache_kernel<T, NT><<<T_, NT, 0, s>>>(a));)
+  }
 }
 
 void launch_gated_group_norm(const float* y, const void* gate, long long ldg, const float* w, int wlen, float eps,
@@ -330,6 +349,9 @@ void launch_gated_group_norm(const float* y, const void* gate, long long ldg, co
   if (group <= 256) {
     DISPATCH_T(f32, (gated_group_norm_kernel<T, 64><<<grid, 64, 0, s>>>(y, (const T*)gate, ldg, w, wlen, eps, group,
                                                                           gate_first, (T*)out, C));)
+  } else if (wide_rows(T_, group)) {
+    DISPATCH_T(f32, (gated_group_norm_kernel<T, 1024><<<grid, 1024, 0, s>>>(y, (const T*)gate, ldg, w, wlen, eps, group,
+                                                                              gate_first, (T*)out, C));)
   } else {
     DISPATCH_T(f32, (gated_group_norm_kernel<T, NT><<<grid, NT, 0, s>>>(y, (const T*)gate, ldg, w, wlen, eps, group,
                                                                           gate_first, (T*)out, C));)

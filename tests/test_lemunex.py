@@ -517,3 +517,38 @@ def test_conv_norm_router_ops(device):
     a = _dev(device, y, dst, ids, wt, h, sh, sg, torch.empty(T_, d))
     ops.moe_mix(a[0], a[1], a[2], a[3], k, E, a[4], a[5], a[6][:, 2:3], a[7])
     assert torch.allclose(a[7].cpu(), want, atol=1e-5)
+
+
+@pytest.mark.parametrize("device", DEVICES)
+def test_row_ops_few_wide_rows(device):
+    """embed_norm, rms_norm_rows, residual_mix_norm and gated_group_norm on a handful of wide rows (the shape of a decode
+    step at real widths, where the kernels use their widest workgroups) and on many narrow ones."""
+    say("op rows wide", device)
+    torch.manual_seed(4)
+    for rows, d in [(3, 1536), (600, 40), (5, 2050)]:
+        eps = 1e-5
+        table, w = torch.randn(50, d), torch.randn(d) * 0.1
+        ids = torch.randint(0, 50, (rows,), dtype=torch.int32)
+        x = torch.empty(rows, d)
+        a = _dev(device, ids, table, w, x)
+        ops.embed_norm(a[0], a[1], a[2], eps, 1.0, a[3])
+        want_x = O.offset_norm(table[ids.long()].double(), w.double(), eps)
+        assert torch.allclose(a[3].cpu(), want_x.float(), atol=1e-5, rtol=1e-5)
+        pick = torch.tensor([rows - 1, 0], dtype=torch.int64)
+        out = torch.empty(2, d)
+        b = _dev(device, pick, out)
+        ops.rms_norm_rows(a[3], b[0], a[2], eps, 1.0, b[1])
+        assert torch.allclose(b[1].cpu(), O.offset_norm(want_x[pick], w.double(), eps).float(), atol=1e-5, rtol=1e-5)
+        p1, p2, p3, bias = torch.randn(rows, d), torch.randn(rows, d), torch.randn(rows, d), torch.randn(d)
+        h = torch.empty(rows, d)
+        c = _dev(device, p1, bias, p2, p3, h)
+        ops.residual_mix_norm(a[3], c[0], 0.6, c[1], c[2], -0.5, c[3], 1.0, a[2], eps, 1.0, c[4])
+        want2 = want_x + 0.6 * (p1.double() + bias.double()) - 0.5 * p2.double() + p3.double()
+        assert torch.allclose(a[3].cpu(), want2.float(), atol=1e-5, rtol=1e-5)
+        assert torch.allclose(c[4].cpu(), O.offset_norm(want2, w.double(), eps).float(), atol=1e-5, rtol=1e-5)
+        y, g, gw = torch.randn(rows, d), torch.randn(rows, d), torch.rand(d) + 0.5
+        s = O.silu(g.double())
+        want3 = (O.unit_rms(y.double() * s, eps) * gw.double()).float()
+        e = _dev(device, y, g, gw, torch.empty(rows, d))
+        ops.gated_group_norm(e[0], e[1], e[2], eps, d, True, e[3])
+        assert torch.allclose(e[3].cpu(), want3, atol=1e-5, rtol=1e-4)
