@@ -21,141 +21,186 @@ SYM_DEV long long cache_row(const int* __restrict__ bt, int kp, int BS, int shif
   return shift >= 0 ? ((long long)bt[kp >> shift] << shift) + (kp & (BS - 1)) : (long long)bt[kp / BS] * BS + kp % BS;
 }
 
-template <typename T>
-SYM_DEV float dot_row(const T* __restrict__ k, const float* __restrict__ q, int dk);
-
-template <>
-SYM_DEV float dot_row<bf16>(const bf16* __restrict__ k, const float* __restrict__ q, int dk) {
-  float acc = 0.f;
-  int e = 0;
-  if ((dk & 7) == 0 && (reinterpret_cast<uintptr_t>(k) & 15) == 0) {
-    for (; e < dk; e += 8) {
-      float f[8];
-      load8(k + e, f);
+// REP dot products of one key row with the REP query vectors of its head group (qs [REP][dk], fp32)
+template <typename T, int REP>
+SYM_DEV void dot_rows(const T* __restrict__ k, const float* __restrict__ qs, int dk, float* out) {
 #pragma unroll
-      for (int i = 0; i < 8; ++i) acc += f[i] * q[e + i];
-    }
-  }
-  for (; e < dk; ++e) acc += (float)k[e] * q[e];
-  return acc;
-}
-
-template <>
-SYM_DEV float dot_row<float>(const float* __restrict__ k, const float* __restrict__ q, int dk) {
-  float acc = 0.f;
+  for (int r = 0; r < REP; ++r) out[r] = 0.f;
   int e = 0;
-  if ((dk & 3) == 0 && (reinterpret_cast<uintptr_t>(k) & 15) == 0) {
-    for (; e < dk; e += 4) {
-      const float4 f = *reinterpret_cast<const float4*>(k + e);
-      acc += f.x * q[e] + f.y * q[e + 1] + f.z * q[e + 2] + f.w * q[e + 3];
+  if constexpr (sizeof(T) == 2) {
+    if ((dk & 7) == 0 && (reinterpret_cast<uintptr_t>(k) & 15) == 0) {
+      for (; e < dk; e += 8) {
+        float f[8];
+        load8(reinterpret_cast<const bf16*>(k) + e, f);
+#pragma unroll
+        for (int r = 0; r < REP; ++r)
+#pragma unroll
+          for (int i = 0; i < 8; ++i) out[r] += f[i] * qs[r * dk + e + i];
+      }
+    }
+  } else {
+    if ((dk & 3) == 0 && (reinterpret_cast<uintptr_t>(k) & 15) == 0) {
+      for (; e < dk; e += 4) {
+        const float4 f = *reinterpret_cast<const float4*>(reinterpret_cast<const float*>(k) + e);
+#pragma unroll
+        for (int r = 0; r < REP; ++r) {
+          const float* q = qs + r * dk + e;
+          out[r] += f.x * q[0] + f.y * q[1] + f.z * q[2] + f.w * q[3];
+        }
+      }
     }
   }
-  for (; e < dk; ++e) acc += k[e] * q[e];
-  return acc;
+  for (; e < dk; ++e) {
+    const float kv = (float)k[e];
+#pragma unroll
+    for (int r = 0; r < REP; ++r) out[r] += kv * qs[r * dk + e];
+  }
 }
 
-// grid (H, T), NW waves.  Wave w walks the key tiles w, w + NW, ... of the row's window with its own running max / sum /
-// accumulator; the waves' partial results meet in LDS at the end (rows of a decode step have few (row, head) pairs
-// and long windows: NW > 1 shortens each wave's walk).  Dynamic LDS: dk + NW * (2 + 64 * MAX_VCOLS) floats.
-template <typename T, int NW>
+// grid (H / REP, T), NW waves.  A workgroup serves REP query heads that share one key / value head (REP = H / G where
+// that is 1, 2, 4 or 8, else 1 with one workgroup per head): a key row is read once for the REP scores, a value row
+// once for the REP accumulators.  Wave w walks the key tiles w, w + NW, ... of the row's window with its own running
+// max / sum / accumulators; the waves' partial results meet in LDS at the end (rows of a decode step have few (row,
+// head) pairs and long windows: NW > 1 shortens each wave's walk).  Dynamic LDS: REP dk + NW REP (2 + 64 nvc) floats.
+template <typename T, int NW, int REP>
 __global__ __launch_bounds__(64 * NW) void window_attn_wave_kernel(WindowAttnArgs a) {
   extern __shared__ float lds[];
-  float* qs = lds;                      // [dk]
-  float* part = lds + a.dk;             // [NW][2 + 64 * MAX_VCOLS]: m, l, acc
-  const int h = blockIdx.x, row = blockIdx.y, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int g = h / (a.H / a.G);
+  float* qs = lds;                      // [REP][dk]
+  float* part = lds + REP * a.dk;       // [NW][REP][2 + 64 nvc]: m, l, acc
+  const int h0 = blockIdx.x * REP, row = blockIdx.y, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int g = h0 / (a.H / a.G);
+  const int nvc = (a.dv + 63) >> 6, pstride = 2 + 64 * nvc;
   const int p = a.positions[row];
   const int j0 = max(0, p - a.window + 1);
   const int* bt = a.block_tables + (long long)a.row_seq[row] * a.max_blocks;
-  const T* q = reinterpret_cast<const T*>(a.q) + ((long long)row * a.H + h) * a.dk;
-  for (int e = threadIdx.x; e < a.dk; e += 64 * NW) qs[e] = (float)q[e] * a.scale;
+  const T* q = reinterpret_cast<const T*>(a.q) + ((long long)row * a.H + h0) * a.dk;   // REP heads: contiguous
+  for (int e = threadIdx.x; e < REP * a.dk; e += 64 * NW) qs[e] = (float)q[e] * a.scale;
   __syncthreads();
   const T* kc = reinterpret_cast<const T*>(a.k_cache);
   const T* vc = reinterpret_cast<const T*>(a.v_cache);
-  float acc[MAX_VCOLS];
+  float acc[REP][MAX_VCOLS];
+  float m[REP], l[REP];
 #pragma unroll
-  for (int i = 0; i < MAX_VCOLS; ++i) acc[i] = 0.f;
-  float m = -INFINITY, l = 0.f;
+  for (int r = 0; r < REP; ++r) {
+    m[r] = -INFINITY, l[r] = 0.f;
+#pragma unroll
+    for (int i = 0; i < MAX_VCOLS; ++i) acc[r][i] = 0.f;
+  }
   for (int t0 = j0 + 64 * wave; t0 <= p; t0 += 64 * NW) {
     const int j = t0 + lane;
-    float s = -INFINITY;
+    float sc[REP], w[REP];
     long long slot = 0;                       // lanes past the row's position: weight 0 on a finite row (slot 0)
     if (j <= p) {
       slot = cache_row(bt, j, a.BS, a.bs_shift);
-      s = dot_row<T>(kc + (slot * a.G + g) * a.dk, qs, a.dk);
+      dot_rows<T, REP>(kc + (slot * a.G + g) * a.dk, qs, a.dk, sc);
     }
-    const float mt = fmaxf(m, wave_max(s));
-    const float w = j <= p ? expf(s - mt) : 0.f;
-    const float corr = expf(m - mt);          // first tile: exp(-inf) = 0 on an all-zero accumulator
-    l = l * corr + wave_sum(w);
-    m = mt;
 #pragma unroll
-    for (int i = 0; i < MAX_VCOLS; ++i) acc[i] *= corr;
+    for (int r = 0; r < REP; ++r) {
+      const float s = j <= p ? sc[r] : -INFINITY;
+      const float mt = fmaxf(m[r], wave_max(s));
+      w[r] = j <= p ? expf(s - mt) : 0.f;
+      const float corr = expf(m[r] - mt);     // first tile: exp(-inf) = 0 on an all-zero accumulator
+      l[r] = l[r] * corr + wave_sum(w[r]);
+      m[r] = mt;
+#pragma unroll
+      for (int i = 0; i < MAX_VCOLS; ++i) acc[r][i] *= corr;
+    }
     const int nt = min(64, p - t0 + 1);
     const int vslot = (int)slot;              // (cache rows fit 31 bits: checked by the op layer)
-    // eight value rows in flight per batch: their cache rows come lane by lane from the scoring phase (no block-table
-    // walk in this loop), the loads of a batch are issued together
-    for (int jj = 0; jj < nt; jj += 8) {
-      float pw[8];
-      const T* vr[8];
+    // value rows VB at a time: their cache rows come lane by lane from the scoring phase (no block-table walk in this
+    // loop), the loads of a batch are issued together and serve all REP heads
+    constexpr int VB = REP >= 4 ? 4 : 8;
+    for (int jj = 0; jj < nt; jj += VB) {
+      float pw[REP][VB];
+      const T* vr[VB];
 #pragma unroll
-      for (int u = 0; u < 8; ++u) {
-        pw[u] = __shfl(w, jj + u, 64);
+      for (int u = 0; u < VB; ++u) {
         vr[u] = vc + ((long long)__shfl(vslot, jj + u, 64) * a.G + g) * a.dv;
+#pragma unroll
+        for (int r = 0; r < REP; ++r) pw[r][u] = __shfl(w[r], jj + u, 64);
       }
 #pragma unroll
       for (int i = 0; i < MAX_VCOLS; ++i) {
         const int c = lane + 64 * i;
         if (c < a.dv) {
-          float vv[8];
+          float vv[VB];
 #pragma unroll
-          for (int u = 0; u < 8; ++u) vv[u] = (float)vr[u][c];
+          for (int u = 0; u < VB; ++u) vv[u] = (float)vr[u][c];
 #pragma unroll
-          for (int u = 0; u < 8; ++u) acc[i] += pw[u] * vv[u];
+          for (int r = 0; r < REP; ++r)
+#pragma unroll
+            for (int u = 0; u < VB; ++u) acc[r][i] += pw[r][u] * vv[u];
         }
       }
     }
   }
   if (NW > 1) {
-    float* mine = part + wave * (2 + 64 * MAX_VCOLS);
-    if (lane == 0) mine[0] = m, mine[1] = l;
 #pragma unroll
-    for (int i = 0; i < MAX_VCOLS; ++i) mine[2 + 64 * i + lane] = acc[i];
+    for (int r = 0; r < REP; ++r) {
+      float* mine = part + (wave * REP + r) * pstride;
+      if (lane == 0) mine[0] = m[r], mine[1] = l[r];
+#pragma unroll
+      for (int i = 0; i < MAX_VCOLS; ++i)
+        if (i < nvc) mine[2 + 64 * i + lane] = acc[r][i];
+    }
     __syncthreads();
     if (wave) return;
-    float M = m;
-    for (int w = 1; w < NW; ++w) M = fmaxf(M, part[w * (2 + 64 * MAX_VCOLS)]);
-    const float f0 = expf(m - M);
-    l *= f0;
 #pragma unroll
-    for (int i = 0; i < MAX_VCOLS; ++i) acc[i] *= f0;
-    for (int w = 1; w < NW; ++w) {
-      const float* o = part + w * (2 + 64 * MAX_VCOLS);
-      const float f = expf(o[0] - M);         // a wave without tiles: exp(-inf) = 0
-      l += o[1] * f;
+    for (int r = 0; r < REP; ++r) {
+      float M = m[r];
+      for (int w2 = 1; w2 < NW; ++w2) M = fmaxf(M, part[(w2 * REP + r) * pstride]);
+      const float f0 = expf(m[r] - M);
+      l[r] *= f0;
 #pragma unroll
-      for (int i = 0; i < MAX_VCOLS; ++i) acc[i] += o[2 + 64 * i + lane] * f;
+      for (int i = 0; i < MAX_VCOLS; ++i) acc[r][i] *= f0;
+      for (int w2 = 1; w2 < NW; ++w2) {
+        const float* o = part + (w2 * REP + r) * pstride;
+        const float f = expf(o[0] - M);       // a wave without tiles: exp(-inf) = 0
+        l[r] += o[1] * f;
+#pragma unroll
+        for (int i = 0; i < MAX_VCOLS; ++i)
+          if (i < nvc) acc[r][i] += o[2 + 64 * i + lane] * f;
+      }
     }
   }
-  float gate = 1.f;
-  if (a.gate) {
-    const float gv = (float)reinterpret_cast<const T*>(a.gate)[(long long)row * a.ldg + h];
-    gate = 1.f / (1.f + expf(-gv));
-  }
-  const float inv = gate / l;
-  T* o = reinterpret_cast<T*>(a.out) + ((long long)row * a.H + h) * a.dv;
 #pragma unroll
-  for (int i = 0; i < MAX_VCOLS; ++i) {
-    const int c = lane + 64 * i;
-    if (c < a.dv) o[c] = (T)(acc[i] * inv);
+  for (int r = 0; r < REP; ++r) {
+    const int h = h0 + r;
+    float gate = 1.f;
+    if (a.gate) {
+      const float gv = (float)reinterpret_cast<const T*>(a.gate)[(long long)row * a.ldg + h];
+      gate = 1.f / (1.f + expf(-gv));
+    }
+    const float inv = gate / l[r];
+    T* o = reinterpret_cast<T*>(a.out) + ((long long)row * a.H + h) * a.dv;
+#pragma unroll
+    for (int i = 0; i < MAX_VCOLS; ++i) {
+      const int c = lane + 64 * i;
+      if (c < a.dv) o[c] = (T)(acc[r][i] * inv);
+    }
   }
+}
+
+template <typename T, int NW, int REP>
+void launch_wave_rep(const WindowAttnArgs& a, hipStream_t s) {
+  dim3 grid(a.H / REP, a.T);
+  const int nvc = (a.dv + 63) / 64;
+  const size_t lds = (size_t)(REP * a.dk + (NW > 1 ? NW * REP * (2 + 64 * nvc) : 0)) * sizeof(float);
+  window_attn_wave_kernel<T, NW, REP><<<grid, 64 * NW, lds, s>>>(a);
 }
 
 template <typename T, int NW>
 void launch_wave(const WindowAttnArgs& a, hipStream_t s) {
-  dim3 grid(a.H, a.T);
-  const size_t lds = (size_t)(a.dk + (NW > 1 ? NW * (2 + 64 * MAX_VCOLS) : 0)) * sizeof(float);
-  window_attn_wave_kernel<T, NW><<<grid, 64 * NW, lds, s>>>(a);
+  // the heads of a key / value group in one workgroup where the group is 2, 4 or 8 heads, the partial results fit LDS and
+  // the groups alone still give the chip a thousand waves (8 rows x 4 groups measured 45 us grouped, 30 us per head;
+  // 64 rows x 8 groups 128 us grouped, 172 us per head)
+  const int rep = a.H / a.G, nvc = (a.dv + 63) / 64;
+  const bool fits = (size_t)(rep * a.dk + NW * rep * (2 + 64 * nvc)) * sizeof(float) <= 60 * 1024 && rep * nvc <= 16 &&
+                    (long long)a.T * a.G * NW >= 1024;
+  if (rep == 8 && fits) launch_wave_rep<T, NW, 8>(a, s);
+  else if (rep == 4 && fits) launch_wave_rep<T, NW, 4>(a, s);
+  else if (rep == 2 && fits) launch_wave_rep<T, NW, 2>(a, s);
+  else launch_wave_rep<T, NW, 1>(a, s);
 }
 
 // ---- tiled kernel for prompt rows (bf16, head sizes DK = DV in {32, 64, 96, 128}) --------------------------------
