@@ -110,8 +110,11 @@ NO_PACKED_FP32 = ["-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
 def build_kernels(verbose: bool = False, force: bool = False) -> str:
     os.makedirs(OBJ, exist_ok=True)
     kdir = os.path.join(CSRC, "kernels")
-    headers = glob.glob(os.path.join(kdir, "*.h")) + glob.glob(os.path.join(kdir, "*.cuh"))
-    sources = sorted(s for s in glob.glob(os.path.join(kdir, "*.hip")) if os.path.basename(s) not in LATENT_KERNELS + HYBRID_KERNELS)
+    # (the family libraries' launcher headers are not included by these translation units)
+    headers = [h for h in glob.glob(os.path.join(kdir, "*.h")) + glob.glob(os.path.join(kdir, "*.cuh"))
+               if os.path.basename(h) not in ("latent_launchers.h", "hybrid_launchers.h")]
+    sources = sorted(s for s in glob.glob(os.path.join(kdir, "*.hip"))
+                     if os.path.basename(s) not in LATENT_KERNELS + HYBRID_KERNELS)
     tinc, tlib, abi = _torch_paths()
     jobs = []
     objs = []
