@@ -247,14 +247,23 @@ __global__ __launch_bounds__(64 * RW) void window_attn_tile_kernel(WindowAttnArg
   float m = -INFINITY, l = 0.f;
   const float sl2 = a.scale * 1.44269504088896341f;
   const int k_lo = max(0, p_first - a.window + 1);
+  // cache blocks of 64 tokens or a multiple: a key tile lies in one block, whose number is read one tile ahead (the
+  // rows' loads then do not wait for a block-table load of their own)
+  const bool one_block = a.bs_shift >= 6;
+  int blk_next = one_block ? bt[(k_lo & ~63) >> a.bs_shift] : 0;
   for (int kt = k_lo & ~63; kt <= p_last; kt += 64) {
+    const long long blk_base = (long long)blk_next << (one_block ? a.bs_shift : 0);
+    if (one_block && kt + 64 <= p_last) blk_next = bt[(kt + 64) >> a.bs_shift];
+    auto row_of = [&](int kp) {
+      return one_block ? blk_base + (kp & (a.BS - 1)) : cache_row(bt, kp, a.BS, a.bs_shift);
+    };
     __syncthreads();                          // every wave is done with the previous tile
     for (int id = threadIdx.x; id < 64 * (DK / 8); id += NTH) {
       const int key = id / (DK / 8), ch = id - key * (DK / 8);
       const int kp = kt + key;
       uint4 v = make_uint4(0, 0, 0, 0);
       if (kp <= p_last) {
-        const long long slot = cache_row(bt, kp, a.BS, a.bs_shift);
+        const long long slot = row_of(kp);
         v = *reinterpret_cast<const uint4*>(kc + (slot * a.G + g) * DK + 8 * ch);
       }
       *reinterpret_cast<uint4*>(Ks + key * KS + 8 * ch) = v;
@@ -268,11 +277,11 @@ __global__ __launch_bounds__(64 * RW) void window_attn_tile_kernel(WindowAttnArg
       va.u = vb.u = make_uint4(0, 0, 0, 0);
       const int kp = kt + key;
       if (kp <= p_last) {
-        const long long slot = cache_row(bt, kp, a.BS, a.bs_shift);
+        const long long slot = row_of(kp);
         va.u = *reinterpret_cast<const uint4*>(vc + (slot * a.G + g) * DV + 8 * ch);
       }
       if (kp + 1 <= p_last) {
-        const long long slot = cache_row(bt, kp + 1, a.BS, a.bs_shift);
+        const long long slot = row_of(kp + 1);
         vb.u = *reinterpret_cast<const uint4*>(vc + (slot * a.G + g) * DV + 8 * ch);
       }
 #pragma unroll
