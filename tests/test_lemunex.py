@@ -23,7 +23,6 @@ from symmetry_amd.engine.sequence import SamplingParams  # noqa: E402
 from symmetry_amd.models import config as C  # noqa: E402
 from symmetry_amd.models.weights import lemunex_random_weights, save_lemunex_checkpoint  # noqa: E402
 
-HAS_GPU = torch.cuda.is_available()
 DEVICES = ["cpu", pytest.param("cuda", marks=pytest.mark.gpu)]
 
 
